@@ -1,0 +1,66 @@
+"""ctypes binding of libarcq_hip.so (the C ABI declared in include/arcq.h).
+
+There is no fallback: if the HIP library has not been built, loading raises and every
+operator with it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libarcq_hip.so")
+HEADER_PATH = os.path.join(_HERE, "..", "include", "arcq.h")
+
+NVFP4 = 0
+MXFP4 = 1
+FORMATS = {"NVFP4": NVFP4, "MXFP4": MXFP4}
+
+_lib = None
+
+
+class ArcqError(RuntimeError):
+    def __init__(self, status: int, where: str):
+        self.status = status
+        msg = lib().arcq_status_string(status).decode()
+        hip = lib().arcq_last_hip_error() if status == 5 else 0
+        super().__init__(f"{where}: {msg} (arcq status {status}" + (f", hipError {hip})" if hip else ")"))
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m arcquant_amd.build` "
+            "(hipcc, --offload-arch=gfx950). arcquant_amd has no non-HIP path.")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, i, f, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+    L.arcq_version.restype = i
+    L.arcq_status_string.argtypes = [i]
+    L.arcq_status_string.restype = ctypes.c_char_p
+    L.arcq_last_hip_error.restype = i
+    L.arcq_group_size.argtypes = [i]
+    L.arcq_group_size.restype = i
+    L.arcq_codes_bytes.argtypes = [i, i, i]
+    L.arcq_codes_bytes.restype = sz
+    L.arcq_scales_bytes.argtypes = [i, i, i, i]
+    L.arcq_scales_bytes.restype = sz
+    quant = [vp, i, i, vp, i, i, f, vp, vp, vp, vp]
+    L.arcq_reorder_quantize_x.argtypes = quant
+    L.arcq_reorder_quantize_w.argtypes = quant
+    L.arcq_rmsnorm_quantize_x.argtypes = [vp, vp, f, i, i, vp, i, i, f, vp, vp, vp, vp]
+    L.arcq_matmul.argtypes = [vp, vp, vp, vp, i, i, i, i, f, vp, vp, vp, vp]
+    L.arcq_check_index.argtypes = [vp, i, vp]
+    L.arcq_dequantize.argtypes = [vp, vp, i, i, i, vp, vp]
+    for name in ("arcq_reorder_quantize_x", "arcq_reorder_quantize_w", "arcq_rmsnorm_quantize_x", "arcq_matmul",
+                 "arcq_check_index", "arcq_dequantize"):
+        getattr(L, name).restype = i
+    _lib = L
+    return L
+
+
+def check(status: int, where: str) -> None:
+    if status != 0:
+        raise ArcqError(status, where)

@@ -1,0 +1,212 @@
+"""Drop-in for the reference's ``agemm`` extension module on PyTorch-ROCm.
+
+Same four operators, same positional arguments and return values as the pybind11 module the
+reference builds from kernels/src/bindings.cpp:547-575:
+
+    matmul(A, B, SFA, SFB, scale)                          -> bf16 [M, N]
+    reorder_quantize_x(X, reorder_index, KE)               -> (QX, SFX)
+    reorder_quantize_w(W, reorder_index, KE)               -> (QW, SFW)
+    rmsnorm_quantize_x(X, W, eps, reorder_index, KE)       -> (QX, SFX)
+
+plus keyword-only extensions the reference does not have:
+
+    fmt="NVFP4" | "MXFP4"   block format (the reference's kernels are NVFP4 only)
+    global_scale            fp32 tensor scale the values are divided by inside the kernel, as
+                            fake_reorder_quantize_x does (model/quantize.py:330); a python
+                            float or a 0-dim CUDA tensor (read on the device, no host sync).
+                            The reference's callers pass X / scale instead, which rounds to
+                            bf16 first (model/qLlamaLayer.py:76).
+
+PyTorch is used for device memory and the current stream only; all arithmetic happens in
+libarcq_hip.so through its C ABI (include/arcq.h).  Errors surface as RuntimeError, like the
+reference's ``std::runtime_error`` (bindings.cpp:157-159).
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import FORMATS, ArcqError  # noqa: F401
+
+__all__ = ["matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "dequantize", "check_index",
+           "unpack_codes", "scale_values"]
+
+
+def _fmt_id(fmt) -> int:
+    try:
+        return FORMATS[fmt] if isinstance(fmt, str) else FORMATS[{0: "NVFP4", 1: "MXFP4"}[int(fmt)]]
+    except KeyError:
+        raise RuntimeError(f"unknown quantization format {fmt!r} (expected 'NVFP4' or 'MXFP4')") from None
+
+
+def _stream(t: torch.Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _require(t: torch.Tensor, name: str, dtype, ndim=None):
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError(f"{name} must be a torch.Tensor")
+    if t.dtype != dtype:
+        raise RuntimeError(f"expected {name} to have dtype {dtype}, but got {t.dtype}")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be on the GPU (got {t.device})")
+    if ndim is not None and t.dim() != ndim:
+        raise RuntimeError(f"{name} must be {ndim}-D (got shape {tuple(t.shape)})")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    return t
+
+
+def _scalar(value, device):
+    """python float / 0-dim tensor -> (host float, device pointer or None, keep-alive)."""
+    if value is None:
+        return 1.0, None, None
+    if isinstance(value, torch.Tensor):
+        if value.numel() != 1:
+            raise RuntimeError("scale must be a scalar")
+        if value.is_cuda:
+            v = value.detach().to(device=device, dtype=torch.float32).reshape(1)
+            return 1.0, ctypes.c_void_p(v.data_ptr()), v
+        return float(value), None, None
+    return float(value), None, None
+
+
+def _quantize(entry, X, gamma, eps, reorder_index, KE, fmt, global_scale):
+    f = _fmt_id(fmt)
+    L = _lib.lib()
+    _require(X, "X", torch.bfloat16, 2)
+    _require(reorder_index, "reorder_index", torch.int16, 1)
+    M, K = X.shape
+    if reorder_index.numel() != K:
+        raise RuntimeError(f"reorder_index has {reorder_index.numel()} entries, expected K={K}")
+    if reorder_index.device != X.device:
+        raise RuntimeError("reorder_index must be on the same device as X")
+    KE = int(KE)
+    G = L.arcq_group_size(f)
+    if K % 32 or K < 32 or K > 32736 or KE < 0 or KE > K or KE % G:
+        raise RuntimeError(f"Value error in {entry}: K={K}, KE={KE} not supported for {fmt} "
+                           f"(need K % 32 == 0, 32 <= K <= 32736, KE % {G} == 0, KE <= K)")
+    gs, d_gs, keep = _scalar(global_scale, X.device)
+    QX = torch.empty((M, (K + KE) // 2), dtype=torch.uint8, device=X.device)
+    SFX = torch.empty((L.arcq_scales_bytes(M, K, KE, f),), dtype=torch.uint8, device=X.device)
+    with torch.cuda.device(X.device):
+        if gamma is None:
+            rc = getattr(L, entry)(X.data_ptr(), M, K, reorder_index.data_ptr(), KE, f, gs, d_gs, QX.data_ptr(),
+                                   SFX.data_ptr(), _stream(X))
+        else:
+            _require(gamma, "W", torch.bfloat16, 1)
+            if gamma.numel() != K or gamma.device != X.device:
+                raise RuntimeError(f"RMSNorm weight must have K={K} entries on X's device")
+            rc = L.arcq_rmsnorm_quantize_x(X.data_ptr(), gamma.data_ptr(), float(eps), M, K,
+                                           reorder_index.data_ptr(), KE, f, gs, d_gs, QX.data_ptr(),
+                                           SFX.data_ptr(), _stream(X))
+    _lib.check(rc, entry)
+    del keep
+    return QX, SFX
+
+
+def reorder_quantize_x(X, reorder_index, KE, *, fmt="NVFP4", global_scale=None):
+    """agemm.reorder_quantize_x (kernels/src/bindings.cpp:122-163).
+    X bf16 [M,K]; reorder_index int16 [K]; returns QX u8 [M,(K+KE)/2], SFX u8 [M*(K+KE)/G]."""
+    return _quantize("arcq_reorder_quantize_x", X, None, 0.0, reorder_index, KE, fmt, global_scale)
+
+
+def reorder_quantize_w(W, reorder_index, KE, *, fmt="NVFP4", global_scale=None):
+    """agemm.reorder_quantize_w (kernels/src/bindings.cpp:170-210)."""
+    return _quantize("arcq_reorder_quantize_w", W, None, 0.0, reorder_index, KE, fmt, global_scale)
+
+
+def rmsnorm_quantize_x(X, W, eps, reorder_index, KE, *, fmt="NVFP4", global_scale=None):
+    """agemm.rmsnorm_quantize_x (kernels/src/bindings.cpp:216-254); W is the RMSNorm weight bf16 [K]."""
+    return _quantize("arcq_rmsnorm_quantize_x", X, W, eps, reorder_index, KE, fmt, global_scale)
+
+
+def _infer_fmt(A, SFA, fmt):
+    if fmt is not None:
+        return _fmt_id(fmt)
+    M, half = A.shape
+    n = SFA.numel()
+    if n == M * (2 * half // 16):
+        return FORMATS["NVFP4"]
+    if n == M * (2 * half // 32):
+        return FORMATS["MXFP4"]
+    raise RuntimeError(f"cannot tell the block format from SFA ({n} scale bytes for {M}x{2 * half} values)")
+
+
+def matmul(A, B, SFA, SFB, scale, *, fmt=None):
+    """agemm.matmul (kernels/src/bindings.cpp:99-120): bf16 [M,N] = scale * dq(A) @ dq(B)^T.
+
+    A u8 [M,K'/2], B u8 [N,K'/2], SFA/SFB as returned by the quantizers.  ``scale`` may be a
+    python float (as in the reference), a 0-dim tensor, or a pair of 0-dim CUDA tensors
+    (scale_x, scale_w) whose product is formed on the device -- the last two avoid the host sync
+    the reference's float argument forces (model/qLinearLayer.py:69).
+    """
+    _require(A, "A", torch.uint8, 2)
+    _require(B, "B", torch.uint8, 2)
+    _require(SFA, "SFA", torch.uint8)
+    _require(SFB, "SFB", torch.uint8)
+    if A.shape[1] != B.shape[1]:
+        raise RuntimeError(f"A and B disagree on K': {2 * A.shape[1]} vs {2 * B.shape[1]}")
+    f = _infer_fmt(A, SFA, fmt)
+    L = _lib.lib()
+    M, N, Kp = A.shape[0], B.shape[0], 2 * A.shape[1]
+    G = L.arcq_group_size(f)
+    if SFA.numel() != M * (Kp // G) or SFB.numel() != N * (Kp // G):
+        raise RuntimeError("scale buffers do not match the code buffers")
+    if Kp % 64:
+        raise RuntimeError(f"Value error in matmul: K'={Kp} must be a multiple of 64")
+    if isinstance(scale, (tuple, list)):
+        sa, sb = scale
+        ha, da, ka = _scalar(sa, A.device)
+        hb, db, kb = _scalar(sb, A.device)
+        alpha = ha * hb
+    else:
+        alpha, da, ka = _scalar(scale, A.device)
+        db, kb = None, None
+    C = torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
+    with torch.cuda.device(A.device):
+        rc = L.arcq_matmul(A.data_ptr(), SFA.data_ptr(), B.data_ptr(), SFB.data_ptr(), M, N, Kp, f, alpha, da, db,
+                           C.data_ptr(), _stream(A))
+    _lib.check(rc, "arcq_matmul")
+    del ka, kb
+    return C
+
+
+# ------------------------------------------------------------------------------------------
+# helpers for tests and debugging (no counterpart in the reference)
+# ------------------------------------------------------------------------------------------
+
+def dequantize(Q, SF, *, fmt):
+    """codes + scale bytes -> fp32 values q*s [rows, K'] on the device."""
+    f = _fmt_id(fmt)
+    _require(Q, "Q", torch.uint8, 2)
+    _require(SF, "SF", torch.uint8)
+    rows, Kp = Q.shape[0], 2 * Q.shape[1]
+    out = torch.empty((rows, Kp), dtype=torch.float32, device=Q.device)
+    with torch.cuda.device(Q.device):
+        rc = _lib.lib().arcq_dequantize(Q.data_ptr(), SF.data_ptr(), rows, Kp, f, out.data_ptr(), _stream(Q))
+    _lib.check(rc, "arcq_dequantize")
+    return out
+
+
+def check_index(reorder_index) -> None:
+    """Raises RuntimeError unless reorder_index (int16, CUDA) is a permutation of 0..K-1."""
+    _require(reorder_index, "reorder_index", torch.int16, 1)
+    with torch.cuda.device(reorder_index.device):
+        rc = _lib.lib().arcq_check_index(reorder_index.data_ptr(), reorder_index.numel(), _stream(reorder_index))
+    _lib.check(rc, "arcq_check_index")
+
+
+def unpack_codes(Q: torch.Tensor) -> torch.Tensor:
+    """u8 [rows, K'/2] -> u8 [rows, K'] of 4-bit codes (element 2j was the low nibble of byte j)."""
+    return torch.stack([Q & 15, Q >> 4], dim=-1).reshape(Q.shape[0], -1)
+
+
+def scale_values(SF: torch.Tensor, *, fmt) -> torch.Tensor:
+    """scale bytes -> fp32 values (NVFP4: (1+(b&7)/8)*2^((b>>3)-9); MXFP4: 2^(b-127))."""
+    b = SF.to(torch.int32)
+    if _fmt_id(fmt) == FORMATS["NVFP4"]:
+        return torch.ldexp(1.0 + (b & 7).float() / 8.0, (b >> 3) - 9)
+    return torch.ldexp(torch.ones_like(b, dtype=torch.float32), b - 127)

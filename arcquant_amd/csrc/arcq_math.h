@@ -1,0 +1,88 @@
+// arcq_math.h -- the scalar arithmetic of the quantizers, written once for device and host.
+//
+// Every routine here is a closed form of one step of the reference's PyTorch fake quantizer
+// (model/quantize.py); the same source is compiled by hipcc into the kernels and by g++ into
+// a host library (csrc/host_math.cpp) so that CPU tests can sweep it exhaustively.
+#ifndef ARCQ_MATH_H_
+#define ARCQ_MATH_H_
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define ARCQ_HD __host__ __device__ __forceinline__
+#else
+#define ARCQ_HD inline
+#endif
+
+namespace arcq {
+
+ARCQ_HD uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+ARCQ_HD float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+ARCQ_HD float bf16_bits_to_f32(uint32_t h) { return u2f(h << 16); }
+
+// float -> bf16 bits, round to nearest even (finite inputs)
+ARCQ_HD uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = f2u(f);
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// quantize_ue4m3 (model/quantize.py:40-49) of t = amax/6 >= 0: clamp to [2e-3, 448], round to
+// nearest even on a 1+3-bit significand, no subnormals (the floor 2e-3 rounds to 2^-9).
+// Returns the scale byte ((e+9)<<3 | m); *s receives the scale value.
+// A zero block needs no special case: 0 -> 1e-9 -> clamp -> 2e-3 in the reference as well.
+ARCQ_HD uint32_t ue4m3_scale(float t, float *s) {
+  t = t < 2e-3f ? 2e-3f : t;
+  t = t > 448.0f ? 448.0f : t;
+  uint32_t b = f2u(t);
+  b += 0x7ffffu + ((b >> 20) & 1u);
+  b &= 0xfff00000u;
+  *s = u2f(b);
+  return (b >> 20) - ((127u - 9u) << 3);
+}
+
+// quantize_ue8m0 (model/quantize.py:54-59) of t = amax/6 >= 0 (0 is replaced by 1e-9 first,
+// quantize.py:185): 2^ceil(fl(log2(fl(t + 1e-9)))), clamped to 2^+-127.
+// With u = fl(t+1e-9) = 2^k (1 + j 2^-23), fl(log2 u) equals k exactly when j = 0 or when
+// log2(1 + j 2^-23) is below half an ulp of the floats just above k, i.e. j <= jmax(p) with
+// 2^p the binade of those floats: jmax = floor(2^(p-1) ln 2) = 0,0,1,2,5,11,22 for p = 0..6.
+// Otherwise the ceiling is k+1.
+ARCQ_HD uint32_t ue8m0_scale(float t, float *s) {
+  if (t == 0.0f) t = 1e-9f;
+  const uint32_t b = f2u(t + 1e-9f);
+  const int k = (int)(b >> 23) - 127;
+  const uint32_t j = b & 0x7fffffu;
+  const int mag = k > 0 ? k : -k - 1;              // floats just above k lie in the binade of mag
+  const int p = mag > 0 ? 31 - __builtin_clz((unsigned)mag) : -1;
+  const uint32_t jmax = p < 2 ? 0u : ((0x160b050201ull >> (8 * (p - 2))) & 0xffu);
+  int e = k + (j > jmax ? 1 : 0);
+  e = e < -127 ? -127 : (e > 127 ? 127 : e);
+  *s = u2f((uint32_t)(e + 127) << 23);             // e = -127 would be a subnormal; unreachable (u >= 1e-9)
+  return (uint32_t)(e + 127);
+}
+
+// quantize_e2m1 (model/quantize.py:14-22) of the exact quotient n: nearest of
+// {0,.5,1,1.5,2,3,4,6} in magnitude; a tie goes to the lower VALUE (argmin keeps the first
+// minimum on the ascending grid): toward zero for n > 0, away from zero for n < 0.
+// Returns sign<<3 | magnitude index, zero always 0.
+ARCQ_HD uint32_t e2m1_code(float n) {
+  const uint32_t b = f2u(n);
+  const uint32_t neg = b >> 31;
+  const uint32_t u = (b & 0x7fffffffu) + neg;      // "u > bits(mid)"  <=>  |n| > mid, or == mid and n < 0
+  uint32_t i = (u > 0x3e800000u) + (u > 0x3f400000u) + (u > 0x3fa00000u) + (u > 0x3fe00000u) +
+               (u > 0x40200000u) + (u > 0x40600000u) + (u > 0x40a00000u);
+  return i ? (i | (neg << 3)) : 0u;
+}
+
+ARCQ_HD float e2m1_value(uint32_t code) {
+  // 0,.5,1,1.5,2,3,4,6: index i >= 2 is 2^((i>>1)-1) * (1 + (i&1)/2); 1 is the subnormal 0.5
+  const uint32_t i = code & 7u;
+  float v = i ? 0.5f : 0.0f;
+  if (i >= 2u) v = u2f(((126u + (i >> 1)) << 23) | ((i & 1u) << 22));
+  return (code & 8u) ? -v : v;
+}
+
+ARCQ_HD float nvfp4_scale_value(uint32_t byte) { return u2f((byte << 20) + ((127u - 9u) << 23)); }
+ARCQ_HD float mxfp4_scale_value(uint32_t byte) { return u2f(byte << 23); }
+
+}  // namespace arcq
+#endif  // ARCQ_MATH_H_

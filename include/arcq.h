@@ -1,0 +1,136 @@
+/*
+ * arcq.h -- C ABI of libarcq_hip.so: ARCQuant's quantized-linear hot path on MI355X (gfx950).
+ *
+ * Four operators, the ones the reference exports from its pybind11 module `agemm`
+ * (kernels/src/bindings.cpp:547-575), take raw device pointers and sizes and return an
+ * arcq_status.  All work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ * null stream) and nothing synchronises with the host, so a caller may enqueue further work
+ * behind it; the reference launches on the legacy default stream and its callers
+ * synchronise after every call (model/qLinearLayer.py:73).
+ *
+ * Numerics follow the reference's PyTorch fake-quant path (model/quantize.py), not its CUDA
+ * kernels: block scale = amax/6 rounded as quantize_ue4m3 / quantize_ue8m0 do, x/scale as a
+ * correctly rounded fp32 division, e2m1 by nearest value with ties toward the lower value,
+ * the residual of the last `select_num` reordered channels kept in fp32 and quantized again.
+ *
+ * Data layout (internal to the quantizer <-> GEMM pair, like the reference's):
+ *   K'      = K + select_num, channel order [K reordered | select_num residual]
+ *   codes   u8 [rows, K'/2], row-major, element 2j in the low nibble of byte j;
+ *           a code is sign<<3 | magnitude index over {0,.5,1,1.5,2,3,4,6}; zero is 0x0
+ *   scales  u8 [rows, K'/G], row-major, G = 16 (NVFP4) or 32 (MXFP4)
+ *           NVFP4 byte b: (1 + (b&7)/8) * 2^((b>>3) - 9)   (= standard E4M3 byte + 16 from 2^-6 up;
+ *                 the extra low binades hold the values quantize_ue4m3 yields below 2^-6)
+ *           MXFP4 byte b: 2^(b - 127)                      (standard E8M0)
+ */
+#ifndef ARCQ_H_
+#define ARCQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  ARCQ_OK = 0,
+  ARCQ_ERR_NULL = 1,     /* a required pointer is NULL */
+  ARCQ_ERR_SHAPE = 2,    /* rows/K/select_num outside what the path defines */
+  ARCQ_ERR_FORMAT = 3,   /* fmt is neither ARCQ_FMT_NVFP4 nor ARCQ_FMT_MXFP4 */
+  ARCQ_ERR_ALIGN = 4,    /* a pointer is not 16-byte aligned */
+  ARCQ_ERR_LAUNCH = 5,   /* the HIP runtime refused the launch (see arcq_last_hip_error) */
+  ARCQ_ERR_INDEX = 6     /* reorder_index is not a permutation of 0..K-1 (arcq_check_index) */
+} arcq_status;
+
+enum { ARCQ_FMT_NVFP4 = 0, ARCQ_FMT_MXFP4 = 1 };
+
+/* Library version (major*10000 + minor*100 + patch). */
+int arcq_version(void);
+const char *arcq_status_string(int status);
+/* hipError_t of the last failed launch on this thread, as an int (0 = none). */
+int arcq_last_hip_error(void);
+
+/* Block size G of a format (16 / 32), or 0 for an unknown format. */
+int arcq_group_size(int fmt);
+/* Output buffer sizes in bytes for `rows` rows of K channels with select_num residual channels.
+ * Replaces get_sfa_buffer_size_in_bytes / get_sfb_buffer_size_in_bytes
+ * (kernels/src/bindings.cpp:83-95) and the QX/QW shape rule (bindings.cpp:133,181). */
+size_t arcq_codes_bytes(int rows, int K, int select_num);
+size_t arcq_scales_bytes(int rows, int K, int select_num, int fmt);
+
+/*
+ * Activation quantizer: gather x[:, reorder_index], divide by the tensor scale, block-quantize,
+ * append the quantized residual of the last select_num channels.
+ * Replaces agemm.reorder_quantize_x (kernels/src/bindings.cpp:122-163; kernels
+ * reorder.cu:68-203, 380-555, down.cu:71-233) with the numerics of fake_reorder_quantize_x
+ * (model/quantize.py:314-343).
+ *   x              bf16 [M,K] row-major, device
+ *   reorder_index  int16 [K], device; a permutation of 0..K-1 (not checked here)
+ *   select_num     multiple of G, 0 <= select_num <= K
+ *   K              multiple of 32, 32 <= K <= 32736 (int16 index range)
+ *   global_scale / d_global_scale: the fp32 tensor scale values are divided by
+ *                  (quantize.py:330).  If d_global_scale != NULL it is read on the device
+ *                  (no host sync) and global_scale is ignored.
+ *   codes, scales  outputs, sizes as arcq_codes_bytes / arcq_scales_bytes
+ */
+int arcq_reorder_quantize_x(const void *x, int M, int K, const int16_t *reorder_index, int select_num, int fmt,
+                            float global_scale, const float *d_global_scale, void *codes, void *scales,
+                            void *stream);
+
+/*
+ * Weight quantizer: same gather and block quantizer; the last select_num channels are
+ * repeated verbatim (codes and scales) instead of a residual.
+ * Replaces agemm.reorder_quantize_w (kernels/src/bindings.cpp:170-210; reorder.cu:210-330,
+ * 562-696, down.cu:240-361) with the numerics of fake_reorder_quantize_w
+ * (model/quantize.py:287-312).
+ */
+int arcq_reorder_quantize_w(const void *w, int N, int K, const int16_t *reorder_index, int select_num, int fmt,
+                            float global_scale, const float *d_global_scale, void *codes, void *scales,
+                            void *stream);
+
+/*
+ * Fused RMSNorm + activation quantizer.
+ * Replaces agemm.rmsnorm_quantize_x (kernels/src/bindings.cpp:216-254; rmsnorm.cu:68-255).
+ * Normalisation is the PyTorch one the reference's layers run before quantizing
+ * (benchmarks/modeling_arc.py:237-242): h = bf16(x * rsqrt(mean(x^2) + eps)) in fp32,
+ * y = bf16(gamma * h); mean(x^2) is the correctly rounded one (fp64 accumulation).
+ *   gamma  bf16 [K], device
+ * The reference's op has no tensor scale (it quantizes y as is); pass global_scale = 1 and
+ * d_global_scale = NULL for that behaviour.
+ */
+int arcq_rmsnorm_quantize_x(const void *x, const void *gamma, float eps, int M, int K,
+                            const int16_t *reorder_index, int select_num, int fmt, float global_scale,
+                            const float *d_global_scale, void *codes, void *scales, void *stream);
+
+/*
+ * Augmented-K block-scaled FP4 GEMM: C[M,N] = alpha * dq(A)[M,K'] @ dq(B)[N,K']^T, fp32
+ * accumulation, bf16 output.
+ * Replaces agemm.matmul (kernels/src/bindings.cpp:99-120 -> nvfp4.cu:35-132).
+ *   a_codes/a_scales  activations as written by the quantizers above, M rows
+ *   b_codes/b_scales  weights, N rows
+ *   Kp                K' = K + select_num, a multiple of 64
+ *   alpha             host factor; if d_alpha_a / d_alpha_b are non-NULL the fp32 values they
+ *                     point to on the device are multiplied in as well (the reference's
+ *                     scale_x * scale_w, model/qLinearLayer.py:69), without a host sync
+ *   c                 bf16 [M,N] row-major
+ */
+int arcq_matmul(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
+                int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b, void *c,
+                void *stream);
+
+/*
+ * Debug helper: checks on the device that reorder_index is a permutation of 0..K-1 and
+ * returns ARCQ_ERR_INDEX otherwise.  Synchronises `stream`.  The reference performs no such
+ * check (kernels/src/reorder.cu:117 indexes shared memory with whatever it is given).
+ */
+int arcq_check_index(const int16_t *reorder_index, int K, void *stream);
+
+/*
+ * Test helper: expands codes+scales to fp32 values q*s, rows x Kp, on the device.
+ */
+int arcq_dequantize(const void *codes, const void *scales, int rows, int Kp, int fmt, float *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARCQ_H_ */

@@ -1,0 +1,66 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every symbol include/arcq.h declares,
+sizes buffers as documented and rejects bad arguments before touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from arcquant_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "arcq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(arcq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = _lib.lib()
+    names = declared_symbols()
+    assert {"arcq_reorder_quantize_x", "arcq_reorder_quantize_w", "arcq_rmsnorm_quantize_x", "arcq_matmul"} <= set(
+        names)
+    for n in names:
+        assert hasattr(L, n), f"{n} is declared in include/arcq.h but not exported"
+    assert L.arcq_version() >= 100
+
+
+def test_buffer_sizes():
+    L = _lib.lib()
+    assert L.arcq_group_size(0) == 16 and L.arcq_group_size(1) == 32 and L.arcq_group_size(7) == 0
+    assert L.arcq_codes_bytes(2048, 4096, 128) == 2048 * 4224 // 2
+    assert L.arcq_scales_bytes(2048, 4096, 128, 0) == 2048 * 4224 // 16
+    assert L.arcq_scales_bytes(2048, 4096, 128, 1) == 2048 * 4224 // 32
+    assert L.arcq_scales_bytes(1, 64, 0, 9) == 0
+
+
+@pytest.mark.parametrize("K,S,fmt,want", [
+    (4096, 128, 2, 3),      # unknown format
+    (4100, 0, 0, 2),        # K not a multiple of 32
+    (16, 0, 0, 2),          # K too small
+    (32768, 0, 0, 2),       # beyond int16 indices
+    (4096, 8, 0, 2),        # select_num not a multiple of the block
+    (4096, 48, 1, 2),       # ... of 32 for MXFP4
+    (4096, 8192, 0, 2),     # select_num > K
+])
+def test_argument_errors_need_no_gpu(K, S, fmt, want):
+    L = _lib.lib()
+    dummy = ctypes.c_void_p(0x1000)
+    for fn in (L.arcq_reorder_quantize_x, L.arcq_reorder_quantize_w):
+        assert fn(dummy, 4, K, dummy, S, fmt, 1.0, None, dummy, dummy, None) == want
+    assert L.arcq_rmsnorm_quantize_x(dummy, dummy, 1e-5, 4, K, dummy, S, fmt, 1.0, None, dummy, dummy, None) == want
+
+
+def test_null_alignment_and_matmul_errors():
+    L = _lib.lib()
+    ok, odd = ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1004)
+    assert L.arcq_reorder_quantize_x(None, 4, 4096, ok, 0, 0, 1.0, None, ok, ok, None) == 1
+    assert L.arcq_reorder_quantize_x(odd, 4, 4096, ok, 0, 0, 1.0, None, ok, ok, None) == 4
+    assert L.arcq_reorder_quantize_x(ok, 0, 4096, ok, 0, 0, 1.0, None, ok, ok, None) == 0   # zero rows: nothing to do
+    assert L.arcq_matmul(ok, ok, ok, ok, 4, 4, 100, 0, 1.0, None, None, ok, None) == 2       # K' % 64
+    assert L.arcq_matmul(ok, ok, ok, ok, 4, 4, 128, 5, 1.0, None, None, ok, None) == 3
+    assert L.arcq_matmul(ok, None, ok, ok, 4, 4, 128, 0, 1.0, None, None, ok, None) == 1
+    assert L.arcq_matmul(ok, ok, ok, ok, 0, 4, 128, 0, 1.0, None, None, ok, None) == 0
+    assert b"16-byte" in L.arcq_status_string(4)

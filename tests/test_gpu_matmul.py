@@ -1,0 +1,111 @@
+"""GPU parity of the augmented-K FP4 GEMM: within 1e-2 relative Frobenius error of
+dequantize-then-matmul in fp32/fp64 (the stated tolerance; bf16 output rounding alone is
+~2e-3), on seeded inputs quantized by the GPU quantizers (themselves bit-exact, see
+test_gpu_quantize.py)."""
+import numpy as np
+import pytest
+import torch
+
+import recipes
+
+pytestmark = pytest.mark.gpu
+FMTS = ["NVFP4", "MXFP4"]
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def agemm():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from arcquant_amd import agemm as m
+    return m
+
+
+def rel_fro(got, want):
+    got, want = got.double(), want.double()
+    return float((got - want).norm() / want.norm())
+
+
+def quantized_pair(agemm, M, N, K, S, fmt, seed):
+    x = recipes.activations(M, K, seed=seed)
+    w = recipes.weights(N, K, seed=seed + 1)
+    idx = recipes.reorder_index(x)
+    gx, gw = recipes.tensor_scale(x, fmt), recipes.tensor_scale(w, fmt)
+    xd, wd, idxd = x.cuda(), w.cuda(), idx.cuda()
+    a, sfa = agemm.reorder_quantize_x(xd, idxd, S, fmt=fmt, global_scale=gx)
+    b, sfb = agemm.reorder_quantize_w(wd, idxd, S, fmt=fmt, global_scale=gw)
+    return (x, w, idx, gx, gw), (a, sfa, b, sfb)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("M,N,K,S", [(1, 128, 256, 64), (16, 256, 512, 0), (37, 200, 1024, 128), (128, 128, 4096, 256),
+                                     (130, 384, 448, 64)])
+def test_matmul_vs_oracle_fp64(agemm, oracle, fmt, M, N, K, S):
+    (x, w, idx, gx, gw), (a, sfa, b, sfb) = quantized_pair(agemm, M, N, K, S, fmt, seed=40 + M + N)
+    print(f"matmul {fmt} M={M} N={N} K={K} S={S}", flush=True)
+    y = agemm.matmul(a, b, sfa, sfb, gx * gw)
+    assert y.shape == (M, N) and y.dtype == torch.bfloat16
+    G = 16 if fmt == "NVFP4" else 32
+    want = oracle.matmul(a.cpu().numpy(), sfa.cpu().numpy().reshape(M, -1), b.cpu().numpy(),
+                         sfb.cpu().numpy().reshape(N, -1), fmt, alpha=gx * gw)
+    assert sfa.numel() == M * (K + S) // G
+    err = rel_fro(y.cpu().float(), torch.from_numpy(want))
+    assert err < TOL, err
+    # elementwise: bf16 rounding of an fp32-accumulated sum
+    assert torch.allclose(y.cpu().float(), torch.from_numpy(want), rtol=2 ** -7, atol=1e-3 * float(np.abs(want).max()))
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_matmul_scale_argument_forms(agemm, fmt):
+    (x, w, idx, gx, gw), (a, sfa, b, sfb) = quantized_pair(agemm, 48, 256, 512, 64, fmt, seed=5)
+    y0 = agemm.matmul(a, b, sfa, sfb, gx * gw)
+    y1 = agemm.matmul(a, b, sfa, sfb, torch.tensor(gx * gw))                       # CPU tensor, like .item()
+    y2 = agemm.matmul(a, b, sfa, sfb, torch.tensor(gx * gw, device="cuda"))        # device scalar, no sync
+    y3 = agemm.matmul(a, b, sfa, sfb, (torch.tensor(gx, device="cuda"), torch.tensor(gw, device="cuda")))
+    assert torch.equal(y0, y1)
+    for y in (y2, y3):
+        assert rel_fro(y.float(), y0.float()) < 1e-2 and torch.allclose(y.float(), y0.float(), rtol=2 ** -6, atol=0)
+    with pytest.raises(RuntimeError):
+        agemm.matmul(a, b[:, :-32], sfa, sfb, 1.0)
+    with pytest.raises(RuntimeError):
+        agemm.matmul(a.float(), b, sfa, sfb, 1.0)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_identity_weights_recover_activations(agemm, oracle, fmt):
+    """W = I on the reordered channels: Y = d * (dq(x) main + residual) with d = dq(1.0) (1.0 for
+    MXFP4, 1.03125 for NVFP4 whose 1/6 block scale rounds to 0.171875): at most two exact
+    products per output, so the fp32 sum is exact and the bf16 result is determined."""
+    M, K, S = 64, 256, 64
+    x = recipes.activations(M, K, seed=12)
+    idx = torch.arange(K).to(torch.int16)
+    w = torch.eye(K).to(torch.bfloat16)
+    a, sfa = agemm.reorder_quantize_x(x.cuda(), idx.cuda(), S, fmt=fmt)
+    b, sfb = agemm.reorder_quantize_w(w.cuda(), idx.cuda(), S, fmt=fmt)
+    y = agemm.matmul(a, b, sfa, sfb, 1.0).cpu().float()
+    dq = oracle.quantize_x(x, idx, S, fmt, 1.0, want_dq=True)["dq"].astype(np.float64)
+    d = {"NVFP4": 1.03125, "MXFP4": 1.0}[fmt]
+    assert np.all(np.diag(oracle.quantize_w(w, idx, 0, fmt, 1.0, want_dq=True)["dq"]) == d)
+    folded = dq[:, :K].copy()
+    folded[:, K - S:] += dq[:, K:]
+    want = torch.from_numpy(folded * d).to(torch.bfloat16).float()
+    assert torch.equal(y, want)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("M,N,K,S", [(512, 4096, 4096, 256), (2048, 6144, 4096, 256), (256, 4096, 14336, 256)])
+def test_matmul_llama_shapes_vs_torch_fp32(agemm, fmt, M, N, K, S):
+    """Benchmark shapes: compare with torch's fp32 matmul of the dequantized operands on the GPU."""
+    (x, w, idx, gx, gw), (a, sfa, b, sfb) = quantized_pair(agemm, M, N, K, S, fmt, seed=3)
+    print(f"matmul {fmt} M={M} N={N} K={K} S={S}", flush=True)
+    y = agemm.matmul(a, b, sfa, sfb, gx * gw)
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        want = (agemm.dequantize(a, sfa, fmt=fmt) @ agemm.dequantize(b, sfb, fmt=fmt).T) * (gx * gw)
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    err = rel_fro(y.float(), want)
+    assert err < TOL, err
+    # and the whole scheme tracks the unquantized product
+    y_true = x.cuda().float() @ w.cuda().float().T
+    assert rel_fro(y.float(), y_true) < 0.2

@@ -1,0 +1,160 @@
+"""GPU parity of the three quantizers against the CPU oracle: packed codes and scale bytes must be
+bit-identical.  Calls go through the Python op surface, i.e. through the C ABI of libarcq_hip.so."""
+import numpy as np
+import pytest
+import torch
+
+import recipes
+
+pytestmark = pytest.mark.gpu
+FMTS = ["NVFP4", "MXFP4"]
+
+
+@pytest.fixture(scope="module")
+def agemm():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from arcquant_amd import agemm as m
+    return m
+
+
+def dev(t):
+    return t.cuda()
+
+
+def compare(tag, got_codes, got_scales, want):
+    gc = got_codes.cpu().numpy()
+    gs = got_scales.cpu().numpy().reshape(want["scales"].shape)
+    bad_c = int((gc != want["codes"]).sum())
+    bad_s = int((gs != want["scales"]).sum())
+    assert gc.shape == want["codes"].shape
+    assert bad_s == 0, f"{tag}: {bad_s} of {gs.size} scale bytes differ; first at {np.argwhere(gs != want['scales'])[:3]}"
+    assert bad_c == 0, f"{tag}: {bad_c} of {gc.size} code bytes differ; first at {np.argwhere(gc != want['codes'])[:3]}"
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("M,K,S", [(1, 4096, 64), (16, 4096, 256), (33, 4096, 0), (256, 4096, 128), (7, 64, 64),
+                                   (5, 14336, 256), (3, 28672, 512), (130, 2048, 2048), (4, 3584, 128)])
+def test_reorder_quantize_x(agemm, oracle, fmt, M, K, S):
+    x = recipes.activations(M, K, seed=1000 + M + K + S)
+    idx = recipes.reorder_index(x)
+    gs = recipes.tensor_scale(x, fmt)
+    want = oracle.quantize_x(x, idx, S, fmt, gs)
+    print(f"reorder_quantize_x {fmt} M={M} K={K} S={S} gscale={gs}", flush=True)
+    q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), S, fmt=fmt, global_scale=gs)
+    compare("host scale", q, sf, want)
+    # same thing with the tensor scale read on the device
+    q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), S, fmt=fmt,
+                                     global_scale=torch.tensor(gs, dtype=torch.float32).cuda())
+    compare("device scale", q, sf, want)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("N,K,S", [(64, 4096, 128), (9, 14336, 256), (257, 512, 64), (16, 4096, 0)])
+def test_reorder_quantize_w(agemm, oracle, fmt, N, K, S):
+    w = recipes.weights(N, K, seed=2000 + N + K + S)
+    idx = recipes.reorder_index(recipes.activations(32, K, seed=5))
+    gs = recipes.tensor_scale(w, fmt)
+    want = oracle.quantize_w(w, idx, S, fmt, gs)
+    print(f"reorder_quantize_w {fmt} N={N} K={K} S={S}", flush=True)
+    q, sf = agemm.reorder_quantize_w(dev(w), dev(idx), S, fmt=fmt, global_scale=gs)
+    compare("w", q, sf, want)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("M,K,S", [(1, 4096, 64), (16, 4096, 256), (256, 4096, 64), (19, 8192, 256), (6, 2048, 0)])
+def test_rmsnorm_quantize_x(agemm, oracle, fmt, M, K, S):
+    x = recipes.activations(M, K, seed=3000 + M + K + S, outlier_frac=0.005, outlier_gain=50.0)
+    if M > 2:
+        x[2] = 0                                                     # a padding token
+    gam = recipes.gamma(K, seed=7)
+    eps = 1e-5
+    normed = oracle.rmsnorm_quantize_x(x, gam, eps, None, 0, fmt, want_normed=True)["normed"]
+    idx = recipes.reorder_index(torch.from_numpy(normed.astype(np.int16)).view(torch.bfloat16))
+    want = oracle.rmsnorm_quantize_x(x, gam, eps, idx, S, fmt, 1.0)
+    print(f"rmsnorm_quantize_x {fmt} M={M} K={K} S={S}", flush=True)
+    q, sf = agemm.rmsnorm_quantize_x(dev(x), dev(gam), eps, dev(idx), S, fmt=fmt)
+    compare("rmsnorm", q, sf, want)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_edge_values(agemm, oracle, fmt):
+    """zeros, ties, tiny and huge blocks, negative-only blocks, bf16 subnormals."""
+    M, K = 8, 256
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(M, K, generator=g)
+    x[0] = 0.0
+    x[1, :64] = torch.tensor([0.25, -0.25, 0.75, -0.75, 1.25, -1.25, 1.75, -1.75, 2.5, -2.5, 3.5, -3.5, 5, -5, 6,
+                              -6] * 4)                               # exact ties under scale 1
+    x[2] *= 1e-4
+    x[3] *= 1e4
+    x[4] = -x[4].abs()
+    x[5, ::2] = 0
+    x[6] = torch.ldexp(torch.ones(K), torch.randint(-30, 8, (K,), generator=g).float())   # powers of two
+    x[7, :32] = 1e-39                                                                       # bf16 subnormal range
+    x = x.to(torch.bfloat16)
+    idx = torch.arange(K).to(torch.int16)
+    for S in (0, 64):
+        for gs in ((1.0, 0.0371) if fmt == "NVFP4" else (1.0,)):
+            want = oracle.quantize_x(x, idx, S, fmt, gs)
+            q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), S, fmt=fmt, global_scale=gs)
+            compare(f"edge S={S} gs={gs}", q, sf, want)
+
+
+def test_large_shape_properties(agemm, oracle):
+    """Benchmark-size input (4096 x 4096, S=256): full comparison for NVFP4 with a tensor scale and,
+    for both formats, properties that need no oracle: the first K codes do not depend on S, and
+    decode(main) + decode(tail) is closer to x than decode(main) on the selected channels."""
+    M, K, S = 4096, 4096, 256
+    x = recipes.activations(M, K, seed=1)
+    idx = recipes.reorder_index(x)
+    xd, idxd = dev(x), dev(idx)
+    gs = recipes.nvfp4_tensor_scale(x)
+    want = oracle.quantize_x(x, idx, S, "NVFP4", gs)
+    q, sf = agemm.reorder_quantize_x(xd, idxd, S, fmt="NVFP4", global_scale=gs)
+    compare("4096x4096 NVFP4", q, sf, want)
+    for fmt in FMTS:
+        g = gs if fmt == "NVFP4" else 1.0
+        qs, sfs = agemm.reorder_quantize_x(xd, idxd, S, fmt=fmt, global_scale=g)
+        q0, sf0 = agemm.reorder_quantize_x(xd, idxd, 0, fmt=fmt, global_scale=g)
+        assert torch.equal(qs[:, :K // 2], q0)
+        G = 16 if fmt == "NVFP4" else 32
+        assert torch.equal(sfs.view(M, -1)[:, :K // G], sf0.view(M, -1))
+        dq = agemm.dequantize(qs, sfs, fmt=fmt)
+        xr = xd[:, idxd.long()].float() / g
+        e_main = (xr[:, K - S:] - dq[:, K - S:K]).abs().mean()
+        e_arc = (xr[:, K - S:] - dq[:, K - S:K] - dq[:, K:]).abs().mean()
+        assert e_arc < 0.25 * e_main
+
+
+def test_dequantize_matches_oracle(agemm, oracle):
+    x = recipes.activations(12, 512, seed=77)
+    idx = recipes.reorder_index(x)
+    for fmt in FMTS:
+        gs = recipes.tensor_scale(x, fmt)
+        want = oracle.quantize_x(x, idx, 64, fmt, gs, want_dq=True)
+        q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), 64, fmt=fmt, global_scale=gs)
+        assert np.array_equal(agemm.dequantize(q, sf, fmt=fmt).cpu().numpy(), want["dq"])
+
+
+def test_errors(agemm):
+    x = dev(recipes.activations(4, 4096, seed=1))
+    idx = dev(torch.arange(4096).to(torch.int16))
+    with pytest.raises(RuntimeError):
+        agemm.reorder_quantize_x(x.float(), idx, 0)                 # dtype
+    with pytest.raises(RuntimeError):
+        agemm.reorder_quantize_x(x[:, :4000], idx[:4000], 0)        # non-contiguous / bad K
+    with pytest.raises(RuntimeError):
+        agemm.reorder_quantize_x(x, idx, 24)                        # select_num alignment
+    with pytest.raises(RuntimeError):
+        agemm.reorder_quantize_x(x, idx.int(), 0)                   # index dtype
+    with pytest.raises(RuntimeError):
+        agemm.reorder_quantize_x(x.cpu(), idx, 0)                   # device
+    with pytest.raises(RuntimeError):
+        agemm.reorder_quantize_x(x, idx, 0, fmt="INT4")
+    bad = idx.clone()
+    bad[3] = bad[4]
+    with pytest.raises(RuntimeError):
+        agemm.check_index(bad)
+    agemm.check_index(idx)
+    q, sf = agemm.reorder_quantize_x(x[:0], idx, 64)               # empty input
+    assert q.shape == (0, (4096 + 64) // 2) and sf.numel() == 0

@@ -1,0 +1,83 @@
+"""CPU sweeps of the kernels' scalar arithmetic (arcquant_amd/csrc/arcq_math.h compiled by g++)
+against the oracle.  What the GPU executes per element is this same source, so a closed form
+that is wrong anywhere on these sweeps would be wrong in the kernels too."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+from arcquant_amd import build as arcq_build
+
+
+@pytest.fixture(scope="module")
+def hm():
+    path = arcq_build.build_hostmath()
+    L = ctypes.CDLL(path)
+    vp, i = ctypes.c_void_p, ctypes.c_int
+    for n in ("arcq_host_ue4m3", "arcq_host_ue8m0", "arcq_host_e2m1"):
+        getattr(L, n).argtypes = [vp, i, vp, vp]
+    L.arcq_host_scale_values.argtypes = [vp, i, i, vp]
+    return L
+
+
+def run(fn, a):
+    a = np.ascontiguousarray(a, np.float32)
+    val = np.empty_like(a)
+    byte = np.empty(a.shape, np.uint8)
+    fn(a.ctypes.data, a.size, val.ctypes.data, byte.ctypes.data)
+    return val, byte
+
+
+def f32_neighbours(center, width):
+    bits = np.asarray(center, np.float32).view(np.int32)[:, None] + np.arange(-width, width + 1, dtype=np.int32)
+    return bits.reshape(-1).view(np.float32)
+
+
+def scale_inputs(seed):
+    rng = np.random.default_rng(seed)
+    pows = np.ldexp(1.0, np.arange(-60, 60)).astype(np.float32)
+    return np.concatenate([
+        f32_neighbours(pows, 300),                                  # every binade edge, +-300 ulps
+        np.exp2(rng.uniform(-40, 12, 400000)).astype(np.float32),   # log-uniform
+        # amax/6 of bf16-valued amax: what main blocks actually produce
+        (np.arange(0x0080, 0x7f80, dtype=np.uint32) << 16).view(np.float32) / np.float32(6.0),
+        np.array([0.0, 1e-9, 2e-3, 448.0, 1e30], np.float32),
+    ]).astype(np.float32)
+
+
+def test_ue4m3_matches_oracle(hm, oracle):
+    t = np.abs(scale_inputs(1))
+    t = t[np.isfinite(t)]
+    val, byte = run(hm.arcq_host_ue4m3, t)
+    ov, ob = oracle.ue4m3(t)
+    assert np.array_equal(val, ov) and np.array_equal(byte, ob)
+
+
+def test_ue8m0_matches_oracle(hm, oracle):
+    t = np.abs(scale_inputs(2))
+    t = t[np.isfinite(t) & (t < 1e30)]
+    val, byte = run(hm.arcq_host_ue8m0, t)
+    ov, ob = oracle.ue8m0(np.where(t == 0, np.float32(1e-9), t))     # the caller's 0 -> 1e-9 is folded in
+    assert np.array_equal(byte, ob)
+    assert np.array_equal(val, ov)
+
+
+def test_e2m1_matches_oracle(hm, oracle):
+    rng = np.random.default_rng(3)
+    ties = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 0.5, 1, 1.5, 2, 3, 4, 6], np.float32)
+    n = np.concatenate([rng.uniform(-8, 8, 500000).astype(np.float32), f32_neighbours(ties, 4),
+                        -f32_neighbours(ties, 4), np.array([0.0, -0.0, 1e-38, -1e-38, 1e-45, -1e-45, 100, -100,
+                                                            2.0 ** 24, -2.0 ** 24], np.float32)])
+    val, code = run(hm.arcq_host_e2m1, n)
+    ov, oc = oracle.e2m1(n)
+    assert np.array_equal(code, oc)
+    assert np.array_equal(val, ov) and not np.signbit(val[code == 0]).any()
+
+
+def test_scale_byte_decoders(hm, oracle):
+    for fmt, rng_ in ((0, range(0, 143)), (1, range(1, 255))):
+        b = np.array(list(rng_), np.uint8)
+        val = np.empty(b.shape, np.float32)
+        hm.arcq_host_scale_values(b.ctypes.data, b.size, fmt, val.ctypes.data)
+        assert np.array_equal(val, oracle.scale_values(b, fmt))
