@@ -81,6 +81,47 @@ ARCQ_HD float e2m1_value(uint32_t code) {
   return (code & 8u) ? -v : v;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Fast encode for COARSE operands.
+//
+// When the value to encode has few significant bits (a bf16 activation with tensor scale 1: 8
+// bits; its ARC residual y - q*s: the same grid), it is either exactly on a rounding boundary
+// s*mid (a 7-bit number) or at least 2^-10 away from it in units of the block scale.  Then an
+// approximate quotient is enough: w = y*r - 2^-13 with r within 2^-21 (relative) of 1/s lands
+//   * strictly below the boundary for an exact tie  -> the lower value, as the reference's argmin,
+//   * on the correct side of it for everything else,
+// and w is never itself a tie, so the hardware's round-to-nearest-even FP4 conversion
+// (v_cvt_scalef32_pk_fp4_f32) returns the reference's code.  Only "-0" needs cleaning up.
+// tests/test_hostmath.py checks this exhaustively over every bf16 value, block scale and
+// perturbed reciprocal, for main blocks and for residual blocks.
+// ---------------------------------------------------------------------------------------------
+constexpr float kCoarseNudge = 1.220703125e-4f;  // 2^-13
+
+// Model of v_cvt_scalef32_pk_fp4_f32 with scale 1 for one element: round to nearest even,
+// saturate at 6, keep the sign bit even on zero.
+ARCQ_HD uint32_t e2m1_rne_hw_model(float w) {
+  const uint32_t b = f2u(w);
+  const uint32_t a = b & 0x7fffffffu;
+  const uint32_t i = (a > 0x3e800000u) + (a >= 0x3f400000u) + (a > 0x3fa00000u) + (a >= 0x3fe00000u) +
+                     (a > 0x40200000u) + (a >= 0x40600000u) + (a > 0x40a00000u);
+  return i | ((b >> 31) << 3);
+}
+
+// 8 packed codes: a nibble 0x8 (negative zero) becomes 0x0, everything else is unchanged
+ARCQ_HD uint32_t drop_negative_zeros(uint32_t x) {
+  const uint32_t t = (x & 0x77777777u) + 0x77777777u;  // bit 3 of a nibble set iff its magnitude != 0
+  return x & (t | 0x77777777u);
+}
+
+// amax/6 for a coarse amax (bf16-valued): correctly rounded quotient from the rounded reciprocal
+// and one exact remainder (checked for all 128 significands in tests/test_hostmath.py)
+ARCQ_HD float div6_coarse(float a) {
+  const float r6 = 0x1.555556p-3f;
+  const float q = a * r6;
+  const float rem = __builtin_fmaf(-6.0f, q, a);
+  return __builtin_fmaf(rem, r6, q);
+}
+
 ARCQ_HD float nvfp4_scale_value(uint32_t byte) { return u2f((byte << 20) + ((127u - 9u) << 23)); }
 ARCQ_HD float mxfp4_scale_value(uint32_t byte) { return u2f(byte << 23); }
 

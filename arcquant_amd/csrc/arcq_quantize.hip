@@ -7,6 +7,7 @@
 // reordered channels ("unit"): a whole NVFP4 block, or half an MXFP4 block whose other half
 // sits in the neighbouring lane (one cross-lane max).
 #include <hip/hip_runtime.h>
+#include <stdlib.h>
 
 #include "arcq_internal.h"
 #include "arcq_math.h"
@@ -15,6 +16,15 @@ namespace arcq {
 namespace {
 
 enum { MODE_X = 0, MODE_W = 1, MODE_NORM = 2 };
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains outstanding
+// global loads and stores (s_waitcnt vmcnt(0)), which would serialise the next row's prefetch
+// and this row's stores with every barrier.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 constexpr int kThreads = 256;
 
 struct QuantParams {
@@ -95,7 +105,7 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(QuantParams p) 
   const int tail0 = (K - S) >> 4;  // first unit whose channels are among the select_num outliers
 
   for (int r = blockIdx.x; r < p.rows; r += gridDim.x) {
-    __syncthreads();  // the previous row has been consumed (first pass: nothing pending)
+    lds_barrier();  // the previous row has been consumed (first pass: nothing pending)
     const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)r * K);
     double ss = 0.0;
     for (int c = tid; c < nvec; c += kThreads) {
@@ -116,14 +126,14 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(QuantParams p) 
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
       if ((tid & 63) == 0) red[tid >> 6] = ss;
-      __syncthreads();
+      lds_barrier();
       double tot = 0.0;
 #pragma unroll
       for (int w = 0; w < kThreads / 64; ++w) tot += red[w];
       const float var = (float)(tot / (double)K);
       rstd = 1.0f / sqrtf(var + p.eps);
     } else {
-      __syncthreads();
+      lds_barrier();
     }
 
     uint8_t *crow = p.codes + (size_t)r * (Kp >> 1);
@@ -160,11 +170,246 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(QuantParams p) 
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Fast kernels for tensor scale 1 (the fused RMSNorm op, MXFP4, and NVFP4 callers that pass
+// global_scale = 1): every operand of the encoder is then exactly a bf16 value or the residual
+// of one, and the coarse encode of arcq_math.h applies -- one fma and half a hardware FP4
+// conversion per element instead of an IEEE division and seven compares.
+//
+// One workgroup per row at a time, one thread per 16-channel unit (blockDim = K/16 rounded up
+// to whole waves), so everything that depends only on the channel -- gather addresses, gamma --
+// lives in registers across rows:
+//   pass 1 (natural order)  global 2 x 128-bit per thread (next row prefetched), [sum of squares
+//                           in fp64, normalise, gamma] -> packed bf16 into the LDS row
+//   pass 2 (reordered)      16 ds_read_u16_d16_hi into registers whose low halves stay zero
+//                           (a bf16 in the high half IS the fp32), amax, scale, encode, 64-bit store
+// ---------------------------------------------------------------------------------------------
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi) {
+  const v2f v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));  // v_cvt_pk_bf16_f32
+}
+
+// 16 coarse values -> 16 codes with block scale s (r ~ 1/s)
+__device__ __forceinline__ uint2 encode_unit_coarse(const float (&y)[16], float r) {
+  float w[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) w[i] = __builtin_fmaf(y[i], r, -kCoarseNudge);
+  uint32_t a = 0u, b = 0u;
+  a = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(a, w[0], w[1], 1.0f, 0);
+  a = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(a, w[2], w[3], 1.0f, 1);
+  a = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(a, w[4], w[5], 1.0f, 2);
+  a = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(a, w[6], w[7], 1.0f, 3);
+  b = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(b, w[8], w[9], 1.0f, 0);
+  b = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(b, w[10], w[11], 1.0f, 1);
+  b = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(b, w[12], w[13], 1.0f, 2);
+  b = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(b, w[14], w[15], 1.0f, 3);
+  return make_uint2(drop_negative_zeros(a), drop_negative_zeros(b));
+}
+
+template <int FMT>
+__device__ __forceinline__ float unit_amax3(const float (&v)[16]) {
+  float a = fmaxf(fabsf(v[0]), fabsf(v[1]));
+#pragma unroll
+  for (int i = 2; i < 16; i += 2) a = fmaxf(fmaxf(a, fabsf(v[i])), fabsf(v[i + 1]));  // v_max3_f32
+  if (FMT == ARCQ_FMT_MXFP4) a = fmaxf(a, __shfl_xor(a, 1));
+  return a;
+}
+
+// reciprocal of a block scale, within 1 ulp (NVFP4: v_rcp_f32) or exact (MXFP4: power of two)
+template <int FMT>
+__device__ __forceinline__ float scale_rcp(float s) {
+  return FMT == ARCQ_FMT_NVFP4 ? __builtin_amdgcn_rcpf(s) : u2f((254u << 23) - f2u(s));
+}
+
+// gamma * h for the two bf16 halves of one register: v_dot2_f32_bf16 with the other half of the
+// gamma operand zeroed gives the exact fp32 product without unpacking h
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b) {
+  float d;
+  asm("v_dot2_f32_bf16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+
+// Sum of one double per lane over the 64 lanes of a wave, in DPP register moves (no LDS round
+// trips): prefix sums inside each row of 16 lanes, then the row totals are passed along.
+// The total ends up in lane 63.
+__device__ __forceinline__ double wave_sum_to_lane63(double v) {
+#define ARCQ_DPP_STEP(ctrl, row_mask)                                                                     \
+  {                                                                                                        \
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);                                                   \
+    const uint32_t lo = __builtin_amdgcn_update_dpp(0u, (uint32_t)b, ctrl, row_mask, 0xf, false);         \
+    const uint32_t hi = __builtin_amdgcn_update_dpp(0u, (uint32_t)(b >> 32), ctrl, row_mask, 0xf, false); \
+    v += __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);                                           \
+  }
+  ARCQ_DPP_STEP(0x111, 0xf)  // row_shr:1  (lanes shifted in from outside the row read as 0)
+  ARCQ_DPP_STEP(0x112, 0xf)  // row_shr:2
+  ARCQ_DPP_STEP(0x114, 0xf)  // row_shr:4
+  ARCQ_DPP_STEP(0x118, 0xf)  // row_shr:8  -> lane 15 of each row holds the row total
+  ARCQ_DPP_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
+  ARCQ_DPP_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave total
+#undef ARCQ_DPP_STEP
+  return v;
+}
+
+template <int FMT, int MODE>
+__global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p) {
+  extern __shared__ uint4 smem[];
+  constexpr int G = FMT == ARCQ_FMT_NVFP4 ? 16 : 32;
+  const int K = p.K, S = p.S, Kp = K + S;
+  uint16_t *row = reinterpret_cast<uint16_t *>(smem);
+  double *red = reinterpret_cast<double *>(row + K);  // one partial sum per wave
+  const int tid = threadIdx.x;
+  const int nunits = K >> 4;                           // == number of working threads
+  const bool active = tid < nunits;
+  const int tail0 = (K - S) >> 4;
+  const int nwaves = (blockDim.x + 63) >> 6;
+  const bool k_pow2 = (K & (K - 1)) == 0;
+  const double inv_k = 1.0 / (double)K;
+
+  // channel-only state, loaded once
+  uint32_t addr[16];
+  uint32_t glo[8], ghi[8];
+  {
+    const uint32_t base = (uint32_t)reinterpret_cast<uintptr_t>(row);
+    uint4 i0 = make_uint4(0, 0, 0, 0), i1 = i0;
+    if (active) {
+      i0 = reinterpret_cast<const uint4 *>(p.idx)[2 * tid];
+      i1 = reinterpret_cast<const uint4 *>(p.idx)[2 * tid + 1];
+    }
+    const uint32_t iw[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) addr[i] = base + 2u * ((iw[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+    if (MODE == MODE_NORM) {
+      uint4 g0 = make_uint4(0, 0, 0, 0), g1 = g0;
+      if (active) {
+        g0 = reinterpret_cast<const uint4 *>(p.gamma)[tid];
+        g1 = reinterpret_cast<const uint4 *>(p.gamma)[tid + nunits];
+      }
+      const uint32_t gw[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        glo[j] = gw[j] & 0xffffu;       // (gamma_even, 0): v_dot2_f32_bf16 with it = gamma_even * h_even, exact
+        ghi[j] = gw[j] & 0xffff0000u;   // (0, gamma_odd)
+      }
+    }
+  }
+  uint32_t yv[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) yv[i] = 0u;  // low halves stay zero: only d16_hi loads write these
+
+  int r = blockIdx.x;
+  uint4 q0 = make_uint4(0, 0, 0, 0), q1 = q0;
+  if (r < p.rows && active) {
+    const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)r * K);
+    q0 = src[tid];
+    q1 = src[tid + nunits];
+  }
+  for (; r < p.rows; r += gridDim.x) {
+    uint4 n0 = q0, n1 = q1;
+    if (r + (int)gridDim.x < p.rows && active) {  // prefetch the next row of this workgroup
+      const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)(r + gridDim.x) * K);
+      n0 = src[tid];
+      n1 = src[tid + nunits];
+    }
+    if (MODE == MODE_NORM) {
+      const uint32_t xw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+      float f[16];
+      double ss = 0.0;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        f[2 * j] = u2f(xw[j] << 16);
+        f[2 * j + 1] = u2f(xw[j] & 0xffff0000u);
+        const double d0 = (double)f[2 * j], d1 = (double)f[2 * j + 1];
+        ss = __builtin_fma(d0, d0, ss);  // exact squares, fp64 accumulation
+        ss = __builtin_fma(d1, d1, ss);
+      }
+      ss = wave_sum_to_lane63(ss);
+      if ((tid & 63) == 63) red[tid >> 6] = ss;
+      lds_barrier();  // partial sums visible; the previous row's gathers are over
+      double tot = 0.0;
+      for (int w = 0; w < nwaves; ++w) tot += red[w];
+      // mean = tot / K, exactly: a power-of-two K is a scaling, anything else an IEEE division
+      const float var = k_pow2 ? (float)(tot * inv_k) : (float)(tot / (double)K);
+      const float rstd = 1.0f / sqrtf(var + p.eps);
+      uint32_t yw[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t h = pack_bf16_rne(f[2 * j] * rstd, f[2 * j + 1] * rstd);
+        yw[j] = pack_bf16_rne(dot2_bf16(h, glo[j]), dot2_bf16(h, ghi[j]));
+      }
+      if (active) {
+        reinterpret_cast<uint4 *>(row)[tid] = make_uint4(yw[0], yw[1], yw[2], yw[3]);
+        reinterpret_cast<uint4 *>(row)[tid + nunits] = make_uint4(yw[4], yw[5], yw[6], yw[7]);
+      }
+    } else {
+      lds_barrier();  // the previous row's gathers are over
+      if (active) {
+        reinterpret_cast<uint4 *>(row)[tid] = q0;
+        reinterpret_cast<uint4 *>(row)[tid + nunits] = q1;
+      }
+    }
+    lds_barrier();
+
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) asm volatile("ds_read_u16_d16_hi %0, %1" : "+v"(yv[i]) : "v"(addr[i]) : "memory");
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+    float y[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) y[i] = u2f(yv[i]);
+
+    uint8_t *crow = p.codes + (size_t)r * (Kp >> 1);
+    uint8_t *srow = p.scales + (size_t)r * (Kp / G);
+    float s;
+    const uint32_t sb = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(div6_coarse(unit_amax3<FMT>(y)), &s)
+                                              : ue8m0_scale(div6_coarse(unit_amax3<FMT>(y)), &s);
+    const uint2 pk = encode_unit_coarse(y, scale_rcp<FMT>(s));
+    if (active) {
+      store_unit<FMT>(crow, srow, tid, pk, sb);
+      if (tid >= tail0) {
+        if (MODE == MODE_W) {
+          store_unit<FMT>(crow, srow, nunits + (tid - tail0), pk, sb);
+        } else {
+          float e[16];
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const uint32_t c = ((i < 8 ? pk.x : pk.y) >> (4 * (i & 7))) & 15u;
+            e[i] = y[i] - e2m1_value(c) * s;  // exact product, one rounding: the fp32 residual
+          }
+          float s2;
+          const uint32_t sb2 = block_scale<FMT>(unit_amax3<FMT>(e), &s2);
+          const uint2 pk2 = encode_unit_coarse(e, scale_rcp<FMT>(s2));
+          store_unit<FMT>(crow, srow, nunits + (tid - tail0), pk2, sb2);
+        }
+      }
+    }
+    q0 = n0;
+    q1 = n1;
+  }
+}
+
+template <int FMT, int MODE>
+int launch_quantize_unit(const QuantParams &p, hipStream_t stream) {
+  const int threads = (((p.K >> 4) + 63) / 64) * 64;
+  const size_t lds = (size_t)p.K * 2 + 16 * sizeof(double);
+  const int waves_per_wg = threads / 64;
+  // ~32 waves per CU resident at most; leave every workgroup a few rows to amortise its set-up
+  int grid = 256 * (32 / waves_per_wg > 0 ? 32 / waves_per_wg : 1);
+  if (const char *e = getenv("ARCQ_QUANT_GRID")) grid = atoi(e);
+  if (grid > p.rows) grid = p.rows;
+  hipLaunchKernelGGL((quantize_rows_unit_kernel<FMT, MODE>), dim3(grid), dim3(threads), lds, stream, p);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
 __global__ void check_index_kernel(const int16_t *idx, int K, int *bad) {
   extern __shared__ uint4 smem[];
   uint32_t *seen = reinterpret_cast<uint32_t *>(smem);
   for (int i = threadIdx.x; i < (K + 31) / 32; i += blockDim.x) seen[i] = 0u;
-  __syncthreads();
+  lds_barrier();
   for (int i = threadIdx.x; i < K; i += blockDim.x) {
     const int v = idx[i];
     if (v < 0 || v >= K) {
@@ -232,6 +477,17 @@ int quantize_entry(int mode, const void *x, const void *gamma, float eps, int ro
   p.K = K;
   p.S = S;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // tensor scale known on the host to be 1: operands are exactly bf16 -> fast kernels
+  if (!d_gscale && gscale == 1.0f && K <= 16384) {
+    if (fmt == ARCQ_FMT_NVFP4) {
+      if (mode == MODE_X) return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_X>(p, st);
+      if (mode == MODE_W) return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_W>(p, st);
+      return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_NORM>(p, st);
+    }
+    if (mode == MODE_X) return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_X>(p, st);
+    if (mode == MODE_W) return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_W>(p, st);
+    return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_NORM>(p, st);
+  }
   if (fmt == ARCQ_FMT_NVFP4) {
     if (mode == MODE_X) return launch_quantize<ARCQ_FMT_NVFP4, MODE_X>(p, st);
     if (mode == MODE_W) return launch_quantize<ARCQ_FMT_NVFP4, MODE_W>(p, st);

@@ -81,3 +81,20 @@ def test_scale_byte_decoders(hm, oracle):
         val = np.empty(b.shape, np.float32)
         hm.arcq_host_scale_values(b.ctypes.data, b.size, fmt, val.ctypes.data)
         assert np.array_equal(val, oracle.scale_values(b, fmt))
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("residual", [0, 1])
+def test_coarse_fast_encode_is_exact(hm, fmt, residual):
+    """approximate quotient + 2^-13 nudge + hardware RNE == the reference's exact-quotient argmin,
+    for every bf16 value x every block scale (x perturbed reciprocals), main blocks and residuals"""
+    hm.arcq_host_check_coarse.restype = ctypes.c_longlong
+    hm.arcq_host_check_coarse.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_longlong)]
+    n = ctypes.c_longlong(0)
+    bad = hm.arcq_host_check_coarse(fmt, residual, ctypes.byref(n))
+    assert n.value > 1_000_000, n.value
+    assert bad == 0, f"{bad} of {n.value} disagree"
+
+
+def test_div6_coarse_is_exact(hm):
+    assert hm.arcq_host_check_div6() == 0
