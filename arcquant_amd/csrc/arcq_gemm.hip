@@ -10,6 +10,9 @@
 // The weight matrix takes the "A" operand slot and the activations the "B" slot, so that a
 // lane ends up holding four consecutive output columns n of one row m and stores 8 bytes.
 #include <hip/hip_runtime.h>
+#include <stdlib.h>
+
+#include <type_traits>
 
 #include "arcq_internal.h"
 #include "arcq_math.h"
@@ -46,6 +49,17 @@ __device__ __forceinline__ float effective_alpha(const GemmParams &p) {
 // One 32x32 accumulator tile -> C.  acc[v] is (n = n0 + 8*(v/4) + 4*(lane/32) + v%4, m = m0 + lane%32).
 __device__ __forceinline__ void store_tile(const GemmParams &p, const v16f &acc, int m0, int n0, int lane, float alpha) {
   const int m = m0 + (lane & 31);
+  if (m0 + 32 <= p.M && n0 + 32 <= p.N && (p.N & 3) == 0) {  // tile fully inside: no per-element checks
+    uint16_t *crow = p.c + (size_t)m * p.N + n0 + 4 * (lane >> 5);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      uint32_t h[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) h[j] = f32_to_bf16_bits(acc[4 * q + j] * alpha);
+      *reinterpret_cast<uint2 *>(crow + 8 * q) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+    }
+    return;
+  }
   if (m >= p.M) return;
   uint16_t *crow = p.c + (size_t)m * p.N;
 #pragma unroll
@@ -178,6 +192,262 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_direct(GemmParams p) {
     for (int j = 0; j < 2; ++j) store_tile(p, acc[i][j], m_base + 32 * j, n_base + 32 * i, lane, alpha);
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Tiled MXFP4 kernel: 256 threads = 2x2 waves, workgroup tile (64*WN) x (64*WM), K step 256.
+// Requires K' % 128 == 0 (scale rows are then dword-aligned and a K step ends on a dword).
+//
+// Global -> LDS goes through LDS-direct loads (global_load_lds_dwordx4 / _dword): no staging
+// registers, a wave's 64 lanes fill consecutive LDS in lane order.  A code-tile row is 128 bytes =
+// 8 chunks of 16 bytes (one MX block each); lane l of a load fetches row l/8 and, instead of
+// chunk l%8, chunk (l%8) ^ ((row>>1)&7): global reads still cover whole 128-byte lines, while the
+// 16 lanes of an MFMA operand read (16 consecutive rows, same chunk) hit 16 different 16-byte
+// bank groups.  The E8M0 bytes of the step (8 per row) travel the same way, 4 bytes per lane.
+// Two LDS stages: the loads of step k+1 are in flight while step k is multiplied.
+// Every vector-memory instruction of the main loop is one of these loads, written as inline asm
+// and waited for explicitly before the barrier -- the compiler's wait-count pass would otherwise
+// put a vmcnt(0) in front of LDS reads and drain the prefetch in the middle of the MFMAs.
+//
+// Inside a K step a lane with half index kh = lane/32 consumes blocks 4*kh .. 4*kh+3 in its four
+// MFMAs, so its four E8M0 bytes are one dword of the row-major scale array and the byte is
+// picked by the instruction's op_sel.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void lds_dma16(const void *g, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_wave_base), "v"(g)
+               : "memory");  // M0 is written; nothing else in these kernels reads it
+}
+
+__device__ __forceinline__ void lds_dma4(const void *g, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(lds_wave_base), "v"(g) : "memory");
+}
+
+__device__ __forceinline__ void wait_dma_and_sync() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// An FP4 operand of the scaled MFMA is 4 registers; the builtin's type has 8, the upper 4 unused.
+__device__ __forceinline__ v8i fp4_operand(uint4 q) {
+  const v4i v = {(int)q.x, (int)q.y, (int)q.z, (int)q.w};
+  return __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1);
+}
+
+template <int WN, int WM>
+__global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
+  constexpr int BN = 64 * WN, BM = 64 * WM;
+  __shared__ uint4 sW[2 * BN * 8], sX[2 * BM * 8];  // code tiles, two stages each
+  __shared__ uint4 sWs[2 * BN], sXs[2 * BM];        // 16 scale bytes per row (two K steps), two stages each
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kbytes = p.Kp >> 1, ksc = p.Kp >> 5;
+
+  // tile of this workgroup: consecutive workgroup ids go to different XCDs (8 of them, each with
+  // its own L2), so hand each XCD a contiguous run of tiles that walk down M for a fixed weight tile
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  const int per_xcd = (total + 7) >> 3;
+  const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (lin >= total) return;
+  const int n_base = (lin / tiles_m) * BN, m_base = (lin % tiles_m) * BM;
+
+  const int nk = (p.Kp + 255) >> 8;
+  const bool short_last = (p.Kp & 255) != 0;  // then the last step has 4 valid blocks (K' % 256 == 128)
+
+  // ---- global -> LDS plan: codes
+  const int ld_row = tid >> 3;                                   // + 32*i
+  const int ld_q = (tid & 7) ^ ((ld_row >> 1) & 7);              // chunk fetched by this lane
+  const uint8_t *wsrc[WN * 2], *xsrc[WM * 2];
+#pragma unroll
+  for (int i = 0; i < WN * 2; ++i)
+    wsrc[i] = p.b_codes + (size_t)min(n_base + 32 * i + ld_row, p.N - 1) * kbytes + ld_q * 16;
+#pragma unroll
+  for (int i = 0; i < WM * 2; ++i)
+    xsrc[i] = p.a_codes + (size_t)min(m_base + 32 * i + ld_row, p.M - 1) * kbytes + ld_q * 16;
+  // ---- scales: a lane fetches 16 bytes = the E8M0 bytes of one row for a PAIR of K steps; one
+  // load instruction covers 64 rows.  Instruction j of the weights goes to wave j%4, of the
+  // activations to wave (j+WN)%4.  If the row ends inside the last pair, the 16-byte window is
+  // shifted back to end at the row end (sc_shift bytes; K' % 128 == 0 makes it a multiple of 4).
+  const int npairs = (nk + 1) >> 1;
+  const int sc_shift = max(0, npairs * 16 - ksc);
+  const uint8_t *wssrc[WN], *xssrc[WM];
+#pragma unroll
+  for (int j = 0; j < WN; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
+#pragma unroll
+  for (int j = 0; j < WM; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
+  const uint32_t lw0 = (uint32_t)reinterpret_cast<uintptr_t>(sW) + wave * 1024;
+  const uint32_t lx0 = (uint32_t)reinterpret_cast<uintptr_t>(sX) + wave * 1024;
+  const uint32_t lws0 = (uint32_t)reinterpret_cast<uintptr_t>(sWs);
+  const uint32_t lxs0 = (uint32_t)reinterpret_cast<uintptr_t>(sXs);
+
+  auto issue = [&](int kt) {
+    const int st = kt & 1;
+    // a short last step has only chunks 0..3: fetch those twice; the products of the absent blocks
+    // are zeroed in compute()
+    const bool clip = short_last && kt == nk - 1;
+    const int koff = kt * 128 - ((clip && ld_q >= 4) ? 64 : 0);
+#pragma unroll
+    for (int i = 0; i < WN * 2; ++i) lds_dma16(wsrc[i] + koff, lw0 + st * (BN * 128) + i * 4096);
+#pragma unroll
+    for (int i = 0; i < WM * 2; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * 4096);
+#ifndef ARCQ_PROBE_NO_SCALE_DMA
+    if ((kt & 1) == 0) {  // scales of steps kt and kt+1
+      const int pair = kt >> 1, sst = pair & 1;
+      const int soff = pair * 16 - (pair == npairs - 1 ? sc_shift : 0);
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        if ((j & 3) == wave) lds_dma16(wssrc[j] + soff, lws0 + sst * (BN * 16) + j * 1024);
+#pragma unroll
+      for (int j = 0; j < WM; ++j)
+        if (((j + WN) & 3) == wave) lds_dma16(xssrc[j] + soff, lxs0 + sst * (BM * 16) + j * 1024);
+    }
+#endif
+  };
+
+  // ---- LDS -> MFMA operands
+  const int r = lane & 31, kh = lane >> 5;
+  const int swz = (r >> 1) & 7;
+  const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;   // wave tile inside the workgroup tile
+  int w_rd[4], x_rd[4];                                                   // chunk index for tile 0, per sub-step
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    w_rd[ks] = (wn0 + r) * 8 + ((4 * kh + ks) ^ swz);
+    x_rd[ks] = (wm0 + r) * 8 + ((4 * kh + ks) ^ swz);
+  }
+  const int ws_rd = (wn0 + r) * 4, xs_rd = (wm0 + r) * 4;                // first dword of the row's 16 scale bytes
+
+  v16f acc[WN][WM];
+#pragma unroll
+  for (int i = 0; i < WN; ++i)
+#pragma unroll
+    for (int j = 0; j < WM; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  // One K step.  TAIL: the short last step (blocks 4..7 absent): lanes with kh = 1 multiply zeros.
+  // The operand reads of sub-step ks+1 are issued before the MFMAs of sub-step ks (two register
+  // sets), so LDS latency hides behind the matrix pipe.
+  auto compute = [&](int kt, auto tail) {
+    constexpr bool TAIL = decltype(tail)::value;
+    const int st = kt & 1, sst = (kt >> 1) & 1;
+    const uint4 *cw = sW + st * (BN * 8), *cx = sX + st * (BM * 8);
+    // this lane's four scale bytes of the step inside the row's 16-byte pair window; a lane whose
+    // blocks are absent (short last step) may point past it and is clamped: its operands are zero
+    const int sdw = min(3, (kt & 1) * 2 + ((kt >> 1) == npairs - 1 ? (sc_shift >> 2) : 0) + kh);
+    const int *cws = reinterpret_cast<const int *>(sWs) + sst * (BN * 4) + sdw;
+    const int *cxs = reinterpret_cast<const int *>(sXs) + sst * (BM * 4) + sdw;
+    int ws[WN], xs[WM];
+    uint4 wq[2][WN], xq[2][WM];
+    auto fetch = [&](int ks, int b) {
+#pragma unroll
+      for (int i = 0; i < WN; ++i) wq[b][i] = cw[w_rd[ks] + i * 256];
+#pragma unroll
+      for (int j = 0; j < WM; ++j) xq[b][j] = cx[x_rd[ks] + j * 256];
+    };
+#pragma unroll
+    for (int i = 0; i < WN; ++i) ws[i] = cws[ws_rd + i * 128];
+#pragma unroll
+    for (int j = 0; j < WM; ++j) xs[j] = cxs[xs_rd + j * 128];
+    fetch(0, 0);
+#define ARCQ_MX_SUBSTEP(KS)                                                                                   \
+  {                                                                                                           \
+    if (KS < 3) fetch(KS + 1, (KS + 1) & 1);                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                        \
+    v8i wf[WN], xf[WM];                                                                                       \
+    _Pragma("unroll") for (int i = 0; i < WN; ++i) {                                                          \
+      uint4 q = wq[KS & 1][i];                                                                                \
+      if (TAIL && kh) q = make_uint4(0, 0, 0, 0);                                                             \
+      wf[i] = fp4_operand(q);                                                                                 \
+    }                                                                                                         \
+    _Pragma("unroll") for (int j = 0; j < WM; ++j) {                                                          \
+      uint4 q = xq[KS & 1][j];                                                                                \
+      if (TAIL && kh) q = make_uint4(0, 0, 0, 0);                                                             \
+      xf[j] = fp4_operand(q);                                                                                 \
+    }                                                                                                         \
+    _Pragma("unroll") for (int i = 0; i < WN; ++i) _Pragma("unroll") for (int j = 0; j < WM; ++j)             \
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[i], xf[j], acc[i][j], 4, 4, KS, ws[i], \
+                                                                     KS, xs[j]);                              \
+    __builtin_amdgcn_sched_barrier(0);                                                                        \
+  }
+    ARCQ_MX_SUBSTEP(0)
+    ARCQ_MX_SUBSTEP(1)
+    ARCQ_MX_SUBSTEP(2)
+    ARCQ_MX_SUBSTEP(3)
+#undef ARCQ_MX_SUBSTEP
+  };
+
+  const int nfull = short_last ? nk - 1 : nk;
+  issue(0);
+  for (int kt = 0; kt < nfull; ++kt) {
+    wait_dma_and_sync();  // stage kt&1 holds step kt; everyone is done with the other stage
+#ifndef ARCQ_PROBE_NO_DMA
+    if (kt + 1 < nk) issue(kt + 1);
+#endif
+#ifndef ARCQ_PROBE_NO_COMPUTE
+    compute(kt, std::false_type{});
+#endif
+  }
+  if (short_last) {
+    wait_dma_and_sync();
+    compute(nk - 1, std::true_type{});
+  }
+
+  const float alpha = effective_alpha(p);
+  if (m_base + BM <= p.M && n_base + BN <= p.N && (p.N & 7) == 0) {
+    // Whole tile inside C: transpose each wave's tile through LDS (free now) so that every store
+    // instruction writes whole rows of the wave tile, 16 bytes per lane.
+    wait_dma_and_sync();  // every wave is done reading operands
+    constexpr int RB = 64 * WN;                       // bytes per row of the wave tile
+    constexpr int LPR = 4 * WN;                       // lanes per row when reading 16 bytes each
+    uint8_t *region = (wave < 2 ? reinterpret_cast<uint8_t *>(sW) : reinterpret_cast<uint8_t *>(sX)) +
+                      (wave & 1) * (32 * WM * RB);
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
+#pragma unroll
+      for (int j = 0; j < WM; ++j) {
+        const int m = 32 * j + r;
+        const int sw = (m & (LPR - 1)) << 1;          // even: keeps 8-byte chunk pairs adjacent
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint32_t h[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) h[e] = f32_to_bf16_bits(acc[i][j][4 * q + e] * alpha);
+          const int c = 8 * i + 2 * q + kh;           // 8-byte chunk of the row
+          *reinterpret_cast<uint2 *>(region + m * RB + ((c ^ sw) << 3)) =
+              make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        }
+      }
+    const int rr = lane / LPR, t = lane % LPR;
+    uint16_t *cbase = p.c + (size_t)(m_base + wm0) * p.N + n_base + wn0 + 8 * t;
+#pragma unroll
+    for (int it = 0; it < (32 * WM * LPR) / 64; ++it) {
+      const int m = it * (64 / LPR) + rr;
+      const int sw = (m & (LPR - 1)) << 1;
+      const uint4 v = *reinterpret_cast<const uint4 *>(region + m * RB + (((2 * t) ^ sw) << 3));
+      *reinterpret_cast<uint4 *>(cbase + (size_t)m * p.N) = v;
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < WN; ++i)
+#pragma unroll
+    for (int j = 0; j < WM; ++j)
+      store_tile(p, acc[i][j], m_base + wm0 + 32 * j, n_base + wn0 + 32 * i, lane, alpha);
+}
+
+template <int WN, int WM>
+int launch_mxfp4_tiled(const GemmParams &p, hipStream_t st) {
+  constexpr int BN = 64 * WN, BM = 64 * WM;
+  const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  const int grid = ((total + 7) / 8) * 8;  // whole groups of 8 so that the XCD split covers every tile
+  hipLaunchKernelGGL((gemm_mxfp4_tiled<WN, WM>), dim3(grid), dim3(256), 0, st, p);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
 }  // namespace
 }  // namespace arcq
 
@@ -204,6 +474,14 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
   p.Kp = Kp;
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 grid((N + kWgN - 1) / kWgN, (M + kWgM - 1) / kWgM);
+  static const int force = getenv("ARCQ_GEMM_KERNEL") ? atoi(getenv("ARCQ_GEMM_KERNEL")) : -1;
+  if (fmt == ARCQ_FMT_MXFP4 && force != 0 && Kp % 128 == 0) {
+    if (force == 44 || (force < 0 && M > 1024)) return launch_mxfp4_tiled<4, 4>(p, st);
+    if (force == 42) return launch_mxfp4_tiled<4, 2>(p, st);
+    if (force == 24) return launch_mxfp4_tiled<2, 4>(p, st);
+    if (force == 22 || (force < 0 && M > 128)) return launch_mxfp4_tiled<2, 2>(p, st);
+    if (force == 21 || force < 0) return launch_mxfp4_tiled<2, 1>(p, st);
+  }
   if (fmt == ARCQ_FMT_MXFP4)
     hipLaunchKernelGGL(gemm_mxfp4_direct, grid, dim3(256), 0, st, p);
   else
