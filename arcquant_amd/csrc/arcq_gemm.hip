@@ -230,6 +230,56 @@ __device__ __forceinline__ void wait_dma_and_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Epilogue shared by the tiled kernels: acc[i][j] is the 32x32 tile (n-tile i, m-tile j) of the
+// wave tile.  ldsA / ldsB: two LDS areas of at least 2*32*WM*64*WN bytes each, free for reuse.
+template <int WN, int WM>
+__device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (&acc)[WN][WM], uint8_t *ldsA,
+                                                     uint8_t *ldsB, int m_base, int n_base, int wave, int lane) {
+  constexpr int BN = 64 * WN, BM = 64 * WM;
+  const int r = lane & 31, kh = lane >> 5;
+  const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;
+  const float alpha = effective_alpha(p);
+  if (m_base + BM <= p.M && n_base + BN <= p.N && (p.N & 7) == 0) {
+    // Whole tile inside C: transpose each wave's tile through LDS (free now) so that every store
+    // instruction writes whole rows of the wave tile, 16 bytes per lane.
+    wait_dma_and_sync();  // every wave is done reading operands
+    constexpr int RB = 64 * WN;                       // bytes per row of the wave tile
+    constexpr int LPR = 4 * WN;                       // lanes per row when reading 16 bytes each
+    uint8_t *region = (wave < 2 ? ldsA : ldsB) + (wave & 1) * (32 * WM * RB);
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
+#pragma unroll
+      for (int j = 0; j < WM; ++j) {
+        const int m = 32 * j + r;
+        const int sw = (m & (LPR - 1)) << 1;          // even: keeps 8-byte chunk pairs adjacent
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint32_t h[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) h[e] = f32_to_bf16_bits(acc[i][j][4 * q + e] * alpha);
+          const int c = 8 * i + 2 * q + kh;           // 8-byte chunk of the row
+          *reinterpret_cast<uint2 *>(region + m * RB + ((c ^ sw) << 3)) =
+              make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        }
+      }
+    const int rr = lane / LPR, t = lane % LPR;
+    uint16_t *cbase = p.c + (size_t)(m_base + wm0) * p.N + n_base + wn0 + 8 * t;
+#pragma unroll
+    for (int it = 0; it < (32 * WM * LPR) / 64; ++it) {
+      const int m = it * (64 / LPR) + rr;
+      const int sw = (m & (LPR - 1)) << 1;
+      const uint4 v = *reinterpret_cast<const uint4 *>(region + m * RB + (((2 * t) ^ sw) << 3));
+      *reinterpret_cast<uint4 *>(cbase + (size_t)m * p.N) = v;
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < WN; ++i)
+#pragma unroll
+    for (int j = 0; j < WM; ++j)
+      store_tile(p, acc[i][j], m_base + wm0 + 32 * j, n_base + wn0 + 32 * i, lane, alpha);
+}
+
 // An FP4 operand of the scaled MFMA is 4 registers; the builtin's type has 8, the upper 4 unused.
 __device__ __forceinline__ v8i fp4_operand(uint4 q) {
   const v4i v = {(int)q.x, (int)q.y, (int)q.z, (int)q.w};
@@ -395,47 +445,226 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
     compute(nk - 1, std::true_type{});
   }
 
-  const float alpha = effective_alpha(p);
-  if (m_base + BM <= p.M && n_base + BN <= p.N && (p.N & 7) == 0) {
-    // Whole tile inside C: transpose each wave's tile through LDS (free now) so that every store
-    // instruction writes whole rows of the wave tile, 16 bytes per lane.
-    wait_dma_and_sync();  // every wave is done reading operands
-    constexpr int RB = 64 * WN;                       // bytes per row of the wave tile
-    constexpr int LPR = 4 * WN;                       // lanes per row when reading 16 bytes each
-    uint8_t *region = (wave < 2 ? reinterpret_cast<uint8_t *>(sW) : reinterpret_cast<uint8_t *>(sX)) +
-                      (wave & 1) * (32 * WM * RB);
+  store_workgroup_tile<WN, WM>(p, acc, reinterpret_cast<uint8_t *>(sW), reinterpret_cast<uint8_t *>(sX), m_base, n_base,
+                               wave, lane);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tiled NVFP4 kernel: same workgroup tiling, LDS-direct loads and LDS layout as the MXFP4 kernel
+// (a 16-byte chunk is two NVFP4 blocks), but the block scales (1+m/8)*2^e have no hardware path:
+// every wave decodes its operands to fp16 in registers -- code value x scale has at most 6
+// significant bits and lies in [2^-10, 2688], exact in fp16 -- and multiplies them with
+// v_mfma_f32_32x32x16_f16.  Since the scale is applied per element, an MFMA K step need not be a
+// block: a lane reads one 16-byte chunk and feeds its four dwords (8 codes each) to four MFMAs,
+// lanes 0-31 from chunk 4*0+cp, lanes 32-63 from chunk 4*1+cp.
+// Decode of 8 codes (one dword): the 3-bit magnitudes index an 8-entry byte table of fp16 HIGH
+// bytes {00,38,3C,3E,40,42,44,46} (the low byte of those fp16 values is zero) through v_perm_b32,
+// the sign bits are or-ed in, bytes are spread to 16-bit lanes, and one packed fp16 multiply
+// applies the block scale: 16 VALU instructions per 8 values.
+// Requires K' % 128 == 0.
+// ---------------------------------------------------------------------------------------------
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+
+// fp16 bits of two NVFP4 scale bytes sitting in bits 7:0 and 23:16: (1+m/8)*2^(e-9) = (b<<7) + 0x1800
+__device__ __forceinline__ uint32_t nv_scale_pair_f16(uint32_t two_bytes) { return (two_bytes << 7) + 0x18001800u; }
+
+// packed fp16 multiply of both halves of a by the LOW (HI=false) or HIGH half of s.  Plain vector
+// code, not inline asm: the compiler folds the broadcast into op_sel and, unlike with asm, keeps
+// the wait states the matrix pipe needs between a VALU write and an MFMA reading that register.
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+template <bool HI>
+__device__ __forceinline__ uint32_t pk_mul_f16_bcast(uint32_t a, uint32_t s) {
+  const v2h av = __builtin_bit_cast(v2h, a), sv = __builtin_bit_cast(v2h, s);
+  const _Float16 k = HI ? sv[1] : sv[0];
+  const v2h kv = {k, k};
+  return __builtin_bit_cast(uint32_t, av * kv);
+}
+
+template <bool HI>
+__device__ __forceinline__ v8h decode8_nvfp4_f16(uint32_t codes, uint32_t scale_pair) {
+  const uint32_t lut_lo = 0x3e3c3800u, lut_hi = 0x46444240u;  // fp16 high bytes of 0,.5,1,1.5 | 2,3,4,6
+  const uint32_t se = codes & 0x07070707u;                    // magnitudes of elements 0,2,4,6
+  const uint32_t so = (codes >> 4) & 0x07070707u;             // 1,3,5,7
+  uint32_t he = __builtin_amdgcn_perm(lut_hi, lut_lo, se);
+  uint32_t ho = __builtin_amdgcn_perm(lut_hi, lut_lo, so);
+  he |= (codes << 4) & 0x80808080u;                           // signs (bit 3 of a nibble -> bit 7 of the byte)
+  ho |= codes & 0x80808080u;
+  v4u d;
+  d[0] = __builtin_amdgcn_perm(ho, he, 0x040c000cu);          // {0, he.b0, 0, ho.b0}: elements 0,1 as fp16
+  d[1] = __builtin_amdgcn_perm(ho, he, 0x050c010cu);
+  d[2] = __builtin_amdgcn_perm(ho, he, 0x060c020cu);
+  d[3] = __builtin_amdgcn_perm(ho, he, 0x070c030cu);
 #pragma unroll
-    for (int i = 0; i < WN; ++i)
+  for (int k = 0; k < 4; ++k) d[k] = pk_mul_f16_bcast<HI>(d[k], scale_pair);
+  return __builtin_bit_cast(v8h, d);
+}
+
+template <int WN, int WM>
+__global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
+  constexpr int BN = 64 * WN, BM = 64 * WM;
+  __shared__ uint4 sW[2 * BN * 8], sX[2 * BM * 8];  // code tiles, two stages each
+  __shared__ uint4 sWs[2 * BN], sXs[2 * BM];        // 16 scale bytes per row per K step, two stages each
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kbytes = p.Kp >> 1, ksc = p.Kp >> 4;
+
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  const int per_xcd = (total + 7) >> 3;
+  const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (lin >= total) return;
+  const int n_base = (lin / tiles_m) * BN, m_base = (lin % tiles_m) * BM;
+
+  const int nk = (p.Kp + 255) >> 8;
+  const bool short_last = (p.Kp & 255) != 0;  // then the last step has chunks 0..3 and 8 scale bytes
+
+  const int ld_row = tid >> 3;
+  const int ld_q = (tid & 7) ^ ((ld_row >> 1) & 7);
+  const uint8_t *wsrc[WN * 2], *xsrc[WM * 2];
 #pragma unroll
-      for (int j = 0; j < WM; ++j) {
-        const int m = 32 * j + r;
-        const int sw = (m & (LPR - 1)) << 1;          // even: keeps 8-byte chunk pairs adjacent
+  for (int i = 0; i < WN * 2; ++i)
+    wsrc[i] = p.b_codes + (size_t)min(n_base + 32 * i + ld_row, p.N - 1) * kbytes + ld_q * 16;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          uint32_t h[4];
+  for (int i = 0; i < WM * 2; ++i)
+    xsrc[i] = p.a_codes + (size_t)min(m_base + 32 * i + ld_row, p.M - 1) * kbytes + ld_q * 16;
+  // scales: one lane = the 16 scale bytes of one row for this K step; instruction j (64 rows) of
+  // the weights goes to wave j%4, of the activations to wave (j+WN)%4.  In a short last step the
+  // window is shifted back by 8 bytes so that it ends with the row.
+  const uint8_t *wssrc[WN], *xssrc[WM];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) h[e] = f32_to_bf16_bits(acc[i][j][4 * q + e] * alpha);
-          const int c = 8 * i + 2 * q + kh;           // 8-byte chunk of the row
-          *reinterpret_cast<uint2 *>(region + m * RB + ((c ^ sw) << 3)) =
-              make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-        }
-      }
-    const int rr = lane / LPR, t = lane % LPR;
-    uint16_t *cbase = p.c + (size_t)(m_base + wm0) * p.N + n_base + wn0 + 8 * t;
+  for (int j = 0; j < WN; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
 #pragma unroll
-    for (int it = 0; it < (32 * WM * LPR) / 64; ++it) {
-      const int m = it * (64 / LPR) + rr;
-      const int sw = (m & (LPR - 1)) << 1;
-      const uint4 v = *reinterpret_cast<const uint4 *>(region + m * RB + (((2 * t) ^ sw) << 3));
-      *reinterpret_cast<uint4 *>(cbase + (size_t)m * p.N) = v;
-    }
-    return;
+  for (int j = 0; j < WM; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
+  const uint32_t lw0 = (uint32_t)reinterpret_cast<uintptr_t>(sW) + wave * 1024;
+  const uint32_t lx0 = (uint32_t)reinterpret_cast<uintptr_t>(sX) + wave * 1024;
+  const uint32_t lws0 = (uint32_t)reinterpret_cast<uintptr_t>(sWs);
+  const uint32_t lxs0 = (uint32_t)reinterpret_cast<uintptr_t>(sXs);
+
+  auto issue = [&](int kt) {
+    const int st = kt & 1;
+    const bool clip = short_last && kt == nk - 1;
+    const int koff = kt * 128 - ((clip && ld_q >= 4) ? 64 : 0);
+    const int soff = kt * 16 - (clip ? 8 : 0);
+#pragma unroll
+    for (int i = 0; i < WN * 2; ++i) lds_dma16(wsrc[i] + koff, lw0 + st * (BN * 128) + i * 4096);
+#pragma unroll
+    for (int i = 0; i < WM * 2; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * 4096);
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+      if ((j & 3) == wave) lds_dma16(wssrc[j] + soff, lws0 + st * (BN * 16) + j * 1024);
+#pragma unroll
+    for (int j = 0; j < WM; ++j)
+      if (((j + WN) & 3) == wave) lds_dma16(xssrc[j] + soff, lxs0 + st * (BM * 16) + j * 1024);
+  };
+
+  const int r = lane & 31, kh = lane >> 5;
+  const int swz = (r >> 1) & 7;
+  const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;
+  int w_rd[4], x_rd[4];
+#pragma unroll
+  for (int cp = 0; cp < 4; ++cp) {
+    w_rd[cp] = (wn0 + r) * 8 + ((4 * kh + cp) ^ swz);
+    x_rd[cp] = (wm0 + r) * 8 + ((4 * kh + cp) ^ swz);
   }
+
+  v16f acc[WN][WM];
 #pragma unroll
   for (int i = 0; i < WN; ++i)
 #pragma unroll
     for (int j = 0; j < WM; ++j)
-      store_tile(p, acc[i][j], m_base + wm0 + 32 * j, n_base + wn0 + 32 * i, lane, alpha);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  // One K step.  TAIL: chunks 4..7 absent -> lanes with kh = 1 contribute zeros.
+  auto compute = [&](int kt, auto tail) {
+    constexpr bool TAIL = decltype(tail)::value;
+    const int st = kt & 1;
+    const uint4 *cw = sW + st * (BN * 8), *cx = sX + st * (BM * 8);
+    // this lane's 8 scale bytes (blocks 8*kh .. 8*kh+7 of the step) as fp16 pairs:
+    // sp[.][0] = blocks (0,2), [1] = (1,3), [2] = (4,6), [3] = (5,7) relative to 8*kh
+    const int sq = TAIL ? 1 : kh;  // short last step: the 8 valid bytes sit in the upper half of the window
+    uint32_t wsp[WN][4], xsp[WM][4];
+#pragma unroll
+    for (int i = 0; i < WN; ++i) {
+      const uint2 b = reinterpret_cast<const uint2 *>(sWs + st * BN + wn0 + r + 32 * i)[sq];
+      wsp[i][0] = nv_scale_pair_f16(b.x & 0x00ff00ffu);
+      wsp[i][1] = nv_scale_pair_f16((b.x >> 8) & 0x00ff00ffu);
+      wsp[i][2] = nv_scale_pair_f16(b.y & 0x00ff00ffu);
+      wsp[i][3] = nv_scale_pair_f16((b.y >> 8) & 0x00ff00ffu);
+    }
+#pragma unroll
+    for (int j = 0; j < WM; ++j) {
+      const uint2 b = reinterpret_cast<const uint2 *>(sXs + st * BM + wm0 + r + 32 * j)[sq];
+      xsp[j][0] = nv_scale_pair_f16(b.x & 0x00ff00ffu);
+      xsp[j][1] = nv_scale_pair_f16((b.x >> 8) & 0x00ff00ffu);
+      xsp[j][2] = nv_scale_pair_f16(b.y & 0x00ff00ffu);
+      xsp[j][3] = nv_scale_pair_f16((b.y >> 8) & 0x00ff00ffu);
+    }
+#pragma unroll
+    for (int cp = 0; cp < 4; ++cp) {
+      // chunk cp of this lane = blocks 2cp, 2cp+1 -> scale pair index: blocks (0,1)->sp[0].lo, sp[1].lo;
+      // (2,3)->sp[0].hi, sp[1].hi; (4,5)->sp[2].lo, sp[3].lo; (6,7)->sp[2].hi, sp[3].hi
+      uint4 wq[WN], xq[WM];
+#pragma unroll
+      for (int i = 0; i < WN; ++i) {
+        wq[i] = cw[w_rd[cp] + i * 256];
+        if (TAIL && kh) wq[i] = make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < WM; ++j) {
+        xq[j] = cx[x_rd[cp] + j * 256];
+        if (TAIL && kh) xq[j] = make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {  // dword d: 8 codes of block 2cp + d/2
+        v8h wf[WN], xf[WM];
+        constexpr int dummy = 0;
+        (void)dummy;
+#pragma unroll
+        for (int i = 0; i < WN; ++i) {
+          const uint32_t c = d == 0 ? wq[i].x : d == 1 ? wq[i].y : d == 2 ? wq[i].z : wq[i].w;
+          const uint32_t sp = wsp[i][(cp >> 1) * 2 + (d >> 1)];
+          wf[i] = (cp & 1) ? decode8_nvfp4_f16<true>(c, sp) : decode8_nvfp4_f16<false>(c, sp);
+        }
+#pragma unroll
+        for (int j = 0; j < WM; ++j) {
+          const uint32_t c = d == 0 ? xq[j].x : d == 1 ? xq[j].y : d == 2 ? xq[j].z : xq[j].w;
+          const uint32_t sp = xsp[j][(cp >> 1) * 2 + (d >> 1)];
+          xf[j] = (cp & 1) ? decode8_nvfp4_f16<true>(c, sp) : decode8_nvfp4_f16<false>(c, sp);
+        }
+#pragma unroll
+        for (int i = 0; i < WN; ++i)
+#pragma unroll
+          for (int j = 0; j < WM; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[i], xf[j], acc[i][j], 0, 0, 0);
+      }
+    }
+  };
+
+  const int nfull = short_last ? nk - 1 : nk;
+  issue(0);
+  for (int kt = 0; kt < nfull; ++kt) {
+    wait_dma_and_sync();
+    if (kt + 1 < nk) issue(kt + 1);
+    compute(kt, std::false_type{});
+  }
+  if (short_last) {
+    wait_dma_and_sync();
+    compute(nk - 1, std::true_type{});
+  }
+  store_workgroup_tile<WN, WM>(p, acc, reinterpret_cast<uint8_t *>(sW), reinterpret_cast<uint8_t *>(sX), m_base, n_base,
+                               wave, lane);
+}
+
+template <int WN, int WM>
+int launch_nvfp4_tiled(const GemmParams &p, hipStream_t st) {
+  constexpr int BN = 64 * WN, BM = 64 * WM;
+  const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  const int grid = ((total + 7) / 8) * 8;
+  hipLaunchKernelGGL((gemm_nvfp4_tiled<WN, WM>), dim3(grid), dim3(256), 0, st, p);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
 }
 
 template <int WN, int WM>
@@ -481,6 +710,12 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
     if (force == 24) return launch_mxfp4_tiled<2, 4>(p, st);
     if (force == 22 || (force < 0 && M > 128)) return launch_mxfp4_tiled<2, 2>(p, st);
     if (force == 21 || force < 0) return launch_mxfp4_tiled<2, 1>(p, st);
+  }
+  if (fmt == ARCQ_FMT_NVFP4 && force != 0 && Kp % 128 == 0) {
+    if (force == 44) return launch_nvfp4_tiled<4, 4>(p, st);
+    if (force == 42 || (force < 0 && M > 1024)) return launch_nvfp4_tiled<4, 2>(p, st);
+    if (force == 22 || (force < 0 && M > 128)) return launch_nvfp4_tiled<2, 2>(p, st);
+    if (force == 21 || force < 0) return launch_nvfp4_tiled<2, 1>(p, st);
   }
   if (fmt == ARCQ_FMT_MXFP4)
     hipLaunchKernelGGL(gemm_mxfp4_direct, grid, dim3(256), 0, st, p);
