@@ -576,7 +576,12 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  // One K step.  TAIL: chunks 4..7 absent -> lanes with kh = 1 contribute zeros.
+  // One K step = 16 MFMA sub-steps (4 chunks x 4 dwords).  TAIL: chunks 4..7 absent -> lanes with
+  // kh = 1 contribute zeros.  Software pipeline inside the wave: while the MFMAs of sub-step s
+  // run in the matrix pipe, the VALU decodes the operands of sub-step s+1 into a second register
+  // set, and the codes of the next chunk are read from LDS one chunk ahead.  The compiler is told
+  // to issue one MFMA, then a slice of the decode, and so on (sched_group_barrier), because a wave
+  // issues in order and back-to-back MFMAs would leave the VALU idle.
   auto compute = [&](int kt, auto tail) {
     constexpr bool TAIL = decltype(tail)::value;
     const int st = kt & 1;
@@ -601,45 +606,60 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
       xsp[j][2] = nv_scale_pair_f16(b.y & 0x00ff00ffu);
       xsp[j][3] = nv_scale_pair_f16((b.y >> 8) & 0x00ff00ffu);
     }
-#pragma unroll
-    for (int cp = 0; cp < 4; ++cp) {
-      // chunk cp of this lane = blocks 2cp, 2cp+1 -> scale pair index: blocks (0,1)->sp[0].lo, sp[1].lo;
-      // (2,3)->sp[0].hi, sp[1].hi; (4,5)->sp[2].lo, sp[3].lo; (6,7)->sp[2].hi, sp[3].hi
-      uint4 wq[WN], xq[WM];
+    uint4 wq[2][WN], xq[2][WM];   // codes of chunk cp (buffer cp&1)
+    v8h wf[2][WN], xf[2][WM];     // decoded operands of sub-step s (buffer s&1)
+    auto fetch = [&](int cp) {
 #pragma unroll
       for (int i = 0; i < WN; ++i) {
-        wq[i] = cw[w_rd[cp] + i * 256];
-        if (TAIL && kh) wq[i] = make_uint4(0, 0, 0, 0);
+        wq[cp & 1][i] = cw[w_rd[cp] + i * 256];
+        if (TAIL && kh) wq[cp & 1][i] = make_uint4(0, 0, 0, 0);
       }
 #pragma unroll
       for (int j = 0; j < WM; ++j) {
-        xq[j] = cx[x_rd[cp] + j * 256];
-        if (TAIL && kh) xq[j] = make_uint4(0, 0, 0, 0);
+        xq[cp & 1][j] = cx[x_rd[cp] + j * 256];
+        if (TAIL && kh) xq[cp & 1][j] = make_uint4(0, 0, 0, 0);
+      }
+    };
+    // dword d of chunk cp holds 8 codes of block 2cp + d/2: scale pair index (cp>>1)*2 + (d>>1),
+    // low half for even cp, high half for odd cp
+    auto decode = [&](int s) {
+      const int cp = s >> 2, d = s & 3, b = s & 1;
+#pragma unroll
+      for (int i = 0; i < WN; ++i) {
+        const uint4 q = wq[cp & 1][i];
+        const uint32_t c = d == 0 ? q.x : d == 1 ? q.y : d == 2 ? q.z : q.w;
+        const uint32_t sp = wsp[i][(cp >> 1) * 2 + (d >> 1)];
+        wf[b][i] = (cp & 1) ? decode8_nvfp4_f16<true>(c, sp) : decode8_nvfp4_f16<false>(c, sp);
       }
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {  // dword d: 8 codes of block 2cp + d/2
-        v8h wf[WN], xf[WM];
-        constexpr int dummy = 0;
-        (void)dummy;
+      for (int j = 0; j < WM; ++j) {
+        const uint4 q = xq[cp & 1][j];
+        const uint32_t c = d == 0 ? q.x : d == 1 ? q.y : d == 2 ? q.z : q.w;
+        const uint32_t sp = xsp[j][(cp >> 1) * 2 + (d >> 1)];
+        xf[b][j] = (cp & 1) ? decode8_nvfp4_f16<true>(c, sp) : decode8_nvfp4_f16<false>(c, sp);
+      }
+    };
+    fetch(0);
+    decode(0);
 #pragma unroll
-        for (int i = 0; i < WN; ++i) {
-          const uint32_t c = d == 0 ? wq[i].x : d == 1 ? wq[i].y : d == 2 ? wq[i].z : wq[i].w;
-          const uint32_t sp = wsp[i][(cp >> 1) * 2 + (d >> 1)];
-          wf[i] = (cp & 1) ? decode8_nvfp4_f16<true>(c, sp) : decode8_nvfp4_f16<false>(c, sp);
-        }
+    for (int s = 0; s < 16; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+      if ((s & 3) == 0 && s < 12) fetch((s >> 2) + 1);  // next chunk's codes, one chunk ahead
+      if (s < 15) decode(s + 1);
 #pragma unroll
-        for (int j = 0; j < WM; ++j) {
-          const uint32_t c = d == 0 ? xq[j].x : d == 1 ? xq[j].y : d == 2 ? xq[j].z : xq[j].w;
-          const uint32_t sp = xsp[j][(cp >> 1) * 2 + (d >> 1)];
-          xf[j] = (cp & 1) ? decode8_nvfp4_f16<true>(c, sp) : decode8_nvfp4_f16<false>(c, sp);
-        }
+      for (int i = 0; i < WN; ++i)
 #pragma unroll
-        for (int i = 0; i < WN; ++i)
+        for (int j = 0; j < WM; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s & 1][i], xf[s & 1][j], acc[i][j], 0, 0, 0);
+      // issue order for this sub-step: LDS reads first, then MFMA / VALU interleaved
+      if ((s & 3) == 0 && s < 12) __builtin_amdgcn_sched_group_barrier(0x100, WN + WM, 0);
 #pragma unroll
-          for (int j = 0; j < WM; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[i], xf[j], acc[i][j], 0, 0, 0);
+      for (int g = 0; g < WN * WM; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, (16 * (WN + WM) + WN * WM - 1) / (WN * WM), 0);
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   const int nfull = short_last ? nk - 1 : nk;
