@@ -723,17 +723,20 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
   p.Kp = Kp;
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 grid((N + kWgN - 1) / kWgN, (M + kWgM - 1) / kWgM);
+  // Tile choice (ARCQ_GEMM_KERNEL=<WN><WM> forces one, 0 forces the direct kernels; for tuning):
+  // few rows of activations -> small tiles so that enough workgroups exist; many -> large tiles
+  // for operand reuse.  K' % 128 != 0 goes to the direct kernels.
   static const int force = getenv("ARCQ_GEMM_KERNEL") ? atoi(getenv("ARCQ_GEMM_KERNEL")) : -1;
   if (fmt == ARCQ_FMT_MXFP4 && force != 0 && Kp % 128 == 0) {
-    if (force == 44 || (force < 0 && M > 1024)) return launch_mxfp4_tiled<4, 4>(p, st);
-    if (force == 42) return launch_mxfp4_tiled<4, 2>(p, st);
+    if (force == 44) return launch_mxfp4_tiled<4, 4>(p, st);
+    if (force == 42 || (force < 0 && M > 1024)) return launch_mxfp4_tiled<4, 2>(p, st);
     if (force == 24) return launch_mxfp4_tiled<2, 4>(p, st);
     if (force == 22 || (force < 0 && M > 128)) return launch_mxfp4_tiled<2, 2>(p, st);
     if (force == 21 || force < 0) return launch_mxfp4_tiled<2, 1>(p, st);
   }
   if (fmt == ARCQ_FMT_NVFP4 && force != 0 && Kp % 128 == 0) {
-    if (force == 44) return launch_nvfp4_tiled<4, 4>(p, st);
-    if (force == 42 || (force < 0 && M > 1024)) return launch_nvfp4_tiled<4, 2>(p, st);
+    if (force == 44 || (force < 0 && M > 1024)) return launch_nvfp4_tiled<4, 4>(p, st);
+    if (force == 42) return launch_nvfp4_tiled<4, 2>(p, st);
     if (force == 22 || (force < 0 && M > 128)) return launch_nvfp4_tiled<2, 2>(p, st);
     if (force == 21 || force < 0) return launch_nvfp4_tiled<2, 1>(p, st);
   }

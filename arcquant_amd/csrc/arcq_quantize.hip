@@ -421,6 +421,21 @@ __global__ void check_index_kernel(const int16_t *idx, int K, int *bad) {
   }
 }
 
+// plain streaming kernel: reads n16_in 16-byte words, writes n16_out of them back (n16_out <= n16_in)
+__global__ __launch_bounds__(256) void stream_probe_kernel(const uint4 *src, uint4 *dst, size_t n16_in, size_t n16_out) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  uint4 acc = make_uint4(0, 0, 0, 0);
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16_in; i += stride) {
+    const uint4 v = src[i];
+    if (i < n16_out) {
+      dst[i] = v;
+    } else {
+      acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
+    }
+  }
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && n16_out) dst[0] = acc;  // keeps the reads alive
+}
+
 template <int FMT>
 __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t *codes, const uint8_t *scales, int rows, int Kp,
                                                          float *out) {
@@ -551,6 +566,17 @@ int arcq_check_index(const int16_t *reorder_index, int K, void *stream) {
   (void)hipFree(d_bad);
   if (e != hipSuccess) return arcq::note_hip_error(e);
   return bad ? ARCQ_ERR_INDEX : ARCQ_OK;
+}
+
+int arcq_stream_probe(const void *src, void *dst, size_t bytes_in, size_t bytes_out, void *stream) {
+  if (!src || !dst) return ARCQ_ERR_NULL;
+  if (bytes_out > bytes_in || (bytes_in & 15) || (bytes_out & 15)) return ARCQ_ERR_SHAPE;
+  if (!arcq::aligned16(src) || !arcq::aligned16(dst)) return ARCQ_ERR_ALIGN;
+  if (bytes_in == 0) return ARCQ_OK;
+  hipLaunchKernelGGL(arcq::stream_probe_kernel, dim3(2048), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), bytes_in / 16, bytes_out / 16);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
 }
 
 int arcq_dequantize(const void *codes, const void *scales, int rows, int Kp, int fmt, float *out, void *stream) {

@@ -130,6 +130,14 @@ int arcq_check_index(const int16_t *reorder_index, int K, void *stream);
  */
 int arcq_dequantize(const void *codes, const void *scales, int rows, int Kp, int fmt, float *out, void *stream);
 
+/*
+ * Measurement helper (no counterpart in the reference): a plain streaming kernel that reads
+ * bytes_in from src and writes the first bytes_out of them to dst (multiples of 16, bytes_out <=
+ * bytes_in).  bench.py times it with the quantizers' read:write ratio as the achievable HBM
+ * ceiling of the box, and the rocprof FETCH_SIZE / WRITE_SIZE readings are calibrated on it.
+ */
+int arcq_stream_probe(const void *src, void *dst, size_t bytes_in, size_t bytes_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
