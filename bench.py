@@ -33,6 +33,10 @@ MFMA_PEAK_TFLOPS = {"MXFP4": 10100.0, "NVFP4": 2500.0, "bf16": 2500.0}   # dense
 
 H, M_TOKENS, SELECT, EPS = 4096, 4096, 256, 1e-5
 FMT = "NVFP4"
+# HBM bytes per launch of the headline kernel on this workload from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (two runs), each scaled by what the same counter reads for arcq_stream_probe moving a known
+# number of bytes (profiles/bench_quantize_and_gemm_kernels.md): 33.76 MB fetched + 10.09 MB written.
+MEASURED_TRAFFIC_BYTES = 43_850_000
 
 
 def quant_bytes(M, K, S, fmt, fused_norm):
@@ -205,12 +209,13 @@ def main():
     probe_ms = loop_time_ms(probe, 100, torch)
     ceiling = (b_in + b_out) / probe_ms / 1e6
     roofline = {"bound": "hbm", "kernel": "quantize_rows_unit_kernel<NVFP4, RMSNORM>", "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
                 "bytes_per_launch": bytes_per_launch, "avg_launch_us": round(kern_ms * 1e3, 2),
                 "streaming_copy_same_bytes": {"us": round(probe_ms * 1e3, 2), "GB/s": round(ceiling, 1),
                                               "frac_of_peak": round(ceiling / HBM_PEAK_GBS, 4)},
                 "note": "algorithmic bytes / (HIP-event time over the timed region / launches); "
-                        "streaming_copy_same_bytes is a plain copy kernel moving the same bytes on this box"}
+                        "streaming_copy_same_bytes is a plain copy kernel moving the same bytes on this box; "
+                        "traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/)"}
 
     # ---------------- other quantize configurations (reported, not the headline) ----------------
     others = {}
