@@ -122,6 +122,64 @@ ARCQ_HD float div6_coarse(float a) {
   return __builtin_fmaf(rem, r6, q);
 }
 
+// Correctly rounded sqrt(a) from an estimate s0 within 1 ulp of it (the hardware's v_sqrt_f32):
+// the two neighbours' exact residuals decide.  a must be normal and finite (no rescaling here).
+ARCQ_HD float sqrt_from_estimate(float a, float s0) {
+  const float lo = u2f(f2u(s0) - 1u), hi = u2f(f2u(s0) + 1u);
+  const float rlo = __builtin_fmaf(-lo, s0, a), rhi = __builtin_fmaf(-hi, s0, a);
+  float s = rlo <= 0.0f ? lo : s0;
+  s = rhi > 0.0f ? hi : s;
+  return s;
+}
+
+// Correctly rounded 1/s from an estimate r0 within 1 ulp of it (v_rcp_f32): the fused
+// Newton/remainder sequence of an IEEE fp32 division with numerator 1, without the range
+// scaling -- s must lie well inside the normal range (2^-60 < s < 2^60).
+ARCQ_HD float rcp_from_estimate(float s, float r0) {
+  const float e = __builtin_fmaf(-s, r0, 1.0f);
+  const float r = __builtin_fmaf(e, r0, r0);
+  float q = r;
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, 1.0f), r, q);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, 1.0f), r, q);
+  // a significand of all ones is the one case where the iteration can settle one ulp low
+  // (1/s lies just above a rounding midpoint); its reciprocal is 2^-(e+1) * (1 + 2^-23)
+  if ((f2u(s) & 0x7fffffu) == 0x7fffffu) q = u2f(0x7f000000u - f2u(s));
+  return q;
+}
+
+// Midpoint between grid magnitudes m and m+1 (m = 0..6): 0.25 0.75 1.25 1.75 2.5 3.5 5
+ARCQ_HD float e2m1_midpoint(uint32_t m) {
+  return m < 4u ? 0.25f + 0.5f * (float)m : (m == 4u ? 2.5f : (m == 5u ? 3.5f : 5.0f));
+}
+
+// The reference's code for y/s when two conversions of approximate quotients just below and just
+// above it disagree (ca, cb: sign | magnitude, magnitudes one apart, midpoint t between them).
+// With n = RN(y/s) the reference picks the larger magnitude iff n > t (y > 0) or n <= -t (y < 0):
+// nearest value, ties toward the lower value (quantize.py:14-22).  B = t*s is exact in fp32 (3 x 4
+// significant bits), and n > t <=> |y| > B, n <= -t <=> |y| >= B: the half-ulp of slack that the
+// rounding of y/s allows around t is, scaled by s, less than the distance from B to its fp32
+// neighbours, so no fp32 |y| other than B itself can fall inside it.
+ARCQ_HD uint32_t e2m1_resolve(float y, float s, uint32_t ca, uint32_t cb) {
+  const uint32_t ma = ca & 7u, mb = cb & 7u;
+  const uint32_t m = ma < mb ? ma : mb;
+  const float B = e2m1_midpoint(m) * s;
+  const uint32_t neg = f2u(y) >> 31;
+  const uint32_t au = (f2u(y) & 0x7fffffffu) + neg;  // negative y: |y| >= B  <=>  bits(|y|) + 1 > bits(B)
+  const uint32_t mag = m + (au > f2u(B) ? 1u : 0u);
+  return mag ? ((neg << 3) | mag) : 0u;
+}
+
+// a/6 for any a: the same three operations; exact for every significand while a and a*2^-25 are
+// normal (checked exhaustively in tests/test_hostmath.py).  Below that the result may be off by an
+// ulp, which no block scale can see: both scale formats map everything under 2^-40 to one value.
+ARCQ_HD float div6_any(float a) { return div6_coarse(a); }
+
+// x/g for a bf16-valued x: q + (x - g*q)*rg with q = x*rg and rg = RN(1/g)
+ARCQ_HD float div_bf16_by(float x, float g, float rg) {
+  const float q = x * rg;
+  return __builtin_fmaf(__builtin_fmaf(-g, q, x), rg, q);
+}
+
 ARCQ_HD float nvfp4_scale_value(uint32_t byte) { return u2f((byte << 20) + ((127u - 9u) << 23)); }
 ARCQ_HD float mxfp4_scale_value(uint32_t byte) { return u2f(byte << 23); }
 

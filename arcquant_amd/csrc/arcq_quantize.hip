@@ -37,6 +37,7 @@ struct QuantParams {
   float gscale;
   float eps;
   int rows, K, S;
+  double inv_k;           // 1/K (MODE_NORM)
 };
 
 // Block scale from the block's amax: t = amax/6 (quantize.py:155 / :184), then the format's rounding.
@@ -209,6 +210,20 @@ __device__ __forceinline__ uint2 encode_unit_coarse(const float (&y)[16], float 
   return make_uint2(drop_negative_zeros(a), drop_negative_zeros(b));
 }
 
+// 16 codes -> their e2m1 values (hardware FP4 -> fp32 convert, exact)
+__device__ __forceinline__ void decode_unit(uint2 pk, float (&q)[16]) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+#define ARCQ_DEC(j, word, sel)                                                      \
+  {                                                                                 \
+    const v2f t = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, sel);        \
+    q[2 * (j)] = t.x;                                                               \
+    q[2 * (j) + 1] = t.y;                                                           \
+  }
+  ARCQ_DEC(0, pk.x, 0) ARCQ_DEC(1, pk.x, 1) ARCQ_DEC(2, pk.x, 2) ARCQ_DEC(3, pk.x, 3)
+  ARCQ_DEC(4, pk.y, 0) ARCQ_DEC(5, pk.y, 1) ARCQ_DEC(6, pk.y, 2) ARCQ_DEC(7, pk.y, 3)
+#undef ARCQ_DEC
+}
+
 template <int FMT>
 __device__ __forceinline__ float unit_amax3(const float (&v)[16]) {
   float a = fmaxf(fabsf(v[0]), fabsf(v[1]));
@@ -236,6 +251,13 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b) {
 // trips): prefix sums inside each row of 16 lanes, then the row totals are passed along.
 // The total ends up in lane 63.
 __device__ __forceinline__ double wave_sum_to_lane63(double v) {
+#define ARCQ_DPP_STEP_BC(ctrl)                                                                \
+  {                                                                                           \
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);                                       \
+    const uint32_t lo = __builtin_amdgcn_update_dpp(0u, (uint32_t)b, ctrl, 0xf, 0xf, true);   \
+    const uint32_t hi = __builtin_amdgcn_update_dpp(0u, (uint32_t)(b >> 32), ctrl, 0xf, 0xf, true); \
+    v += __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);                               \
+  }
 #define ARCQ_DPP_STEP(ctrl, row_mask)                                                                     \
   {                                                                                                        \
     const uint64_t b = __builtin_bit_cast(uint64_t, v);                                                   \
@@ -243,30 +265,118 @@ __device__ __forceinline__ double wave_sum_to_lane63(double v) {
     const uint32_t hi = __builtin_amdgcn_update_dpp(0u, (uint32_t)(b >> 32), ctrl, row_mask, 0xf, false); \
     v += __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);                                           \
   }
-  ARCQ_DPP_STEP(0x111, 0xf)  // row_shr:1  (lanes shifted in from outside the row read as 0)
-  ARCQ_DPP_STEP(0x112, 0xf)  // row_shr:2
-  ARCQ_DPP_STEP(0x114, 0xf)  // row_shr:4
-  ARCQ_DPP_STEP(0x118, 0xf)  // row_shr:8  -> lane 15 of each row holds the row total
+  ARCQ_DPP_STEP_BC(0x111)    // row_shr:1  (lanes shifted in from outside the row read as 0)
+  ARCQ_DPP_STEP_BC(0x112)    // row_shr:2
+  ARCQ_DPP_STEP_BC(0x114)    // row_shr:4
+  ARCQ_DPP_STEP_BC(0x118)    // row_shr:8  -> lane 15 of each row holds the row total
   ARCQ_DPP_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
   ARCQ_DPP_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave total
 #undef ARCQ_DPP_STEP
+#undef ARCQ_DPP_STEP_BC
   return v;
 }
 
-template <int FMT, int MODE>
+// Two-sided encode for operands that are not coarse (tensor scale not a power of two): the block
+// is converted twice with the hardware RNE convert, from y*r*(1+2^-20) and y*r*(1-2^-20) with
+// r ~ 1/s.  The true quotient y/s, its fp32 rounding and every point where the reference's decision
+// changes differ by far less than 2^-20 relatively, so where the two conversions agree no decision
+// point lies between them and both equal the reference's code.  Where they differ (a few elements
+// in 10^4; exact ties are built into the NVFP4 tensor scale max/2688 = max/(2^7*3*7)) e2m1_resolve
+// decides that element from one exact product.
+__device__ __forceinline__ uint32_t resolve_word(float v0, float v1, float v2, float v3, float v4, float v5, float v6,
+                                                 float v7, float s, uint32_t a, uint32_t b) {
+  uint32_t out = drop_negative_zeros(a);
+  uint32_t d = a ^ b;
+  while (d) {  // one pass per differing element of this lane
+    const int nib = __builtin_ctz(d) >> 2;
+    const float a0 = (nib & 1) ? v1 : v0, a1 = (nib & 1) ? v3 : v2;  // the values are passed one by one
+    const float a2 = (nib & 1) ? v5 : v4, a3 = (nib & 1) ? v7 : v6;  // so that they stay in registers
+    const float b0 = (nib & 2) ? a1 : a0, b1 = (nib & 2) ? a3 : a2;
+    const float yi = (nib & 4) ? b1 : b0;
+    const uint32_t sh = 4u * (uint32_t)nib;
+    const uint32_t c = e2m1_resolve(yi, s, (a >> sh) & 15u, (b >> sh) & 15u);
+    out = (out & ~(15u << sh)) | (c << sh);
+    d &= ~(15u << sh);
+  }
+  return out;
+}
+
+__device__ __forceinline__ uint2 encode_unit_two_sided(const float (&y)[16], float s, float r) {
+  const float ra = r * 0x1.00001p+0f, rb = r * 0x1.ffffep-1f;
+  uint32_t a0 = 0u, a1 = 0u, b0 = 0u, b1 = 0u;
+#define ARCQ_ENC2(dst, rr, i, sel) \
+  dst = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(dst, y[i] * rr, y[i + 1] * rr, 1.0f, sel);
+  ARCQ_ENC2(a0, ra, 0, 0) ARCQ_ENC2(a0, ra, 2, 1) ARCQ_ENC2(a0, ra, 4, 2) ARCQ_ENC2(a0, ra, 6, 3)
+  ARCQ_ENC2(a1, ra, 8, 0) ARCQ_ENC2(a1, ra, 10, 1) ARCQ_ENC2(a1, ra, 12, 2) ARCQ_ENC2(a1, ra, 14, 3)
+  ARCQ_ENC2(b0, rb, 0, 0) ARCQ_ENC2(b0, rb, 2, 1) ARCQ_ENC2(b0, rb, 4, 2) ARCQ_ENC2(b0, rb, 6, 3)
+  ARCQ_ENC2(b1, rb, 8, 0) ARCQ_ENC2(b1, rb, 10, 1) ARCQ_ENC2(b1, rb, 12, 2) ARCQ_ENC2(b1, rb, 14, 3)
+#undef ARCQ_ENC2
+  return make_uint2(resolve_word(y[0], y[1], y[2], y[3], y[4], y[5], y[6], y[7], s, a0, b0),
+                    resolve_word(y[8], y[9], y[10], y[11], y[12], y[13], y[14], y[15], s, a1, b1));
+}
+
+// amax values for which the division-free arithmetic above is not trusted (results that
+// underflow or overflow on the way): everything but zero and the comfortable normal range
+__device__ __forceinline__ bool amax_needs_exact(float a) {
+  return !(a == 0.0f || (a >= 0x1p-100f && a <= 0x1p+120f));
+}
+
+// One unit with IEEE divisions throughout, from the raw bf16 operands: what the reference's
+// arithmetic prescribes literally (quantize.py:154-161, 330, 337-340).
+template <int FMT, bool WITH_RESID>
+__device__ __forceinline__ void unit_exact(const uint32_t (&yv)[16], float g, uint2 *pk, uint32_t *sb, uint2 *pk2,
+                                           uint32_t *sb2) {
+  float v[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) v[i] = u2f(yv[i]) / g;
+  float s;
+  *sb = block_scale<FMT>(unit_amax<FMT>(v), &s);
+  if (!WITH_RESID) {
+    *pk = encode_unit<FMT, false>(v, s);
+  } else {
+    *pk = encode_unit<FMT, true>(v, s);
+    *sb2 = block_scale<FMT>(unit_amax<FMT>(v), &s);
+    *pk2 = encode_unit<FMT, false>(v, s);
+  }
+}
+
+template <int FMT, int MODE, bool SCALED>
 __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p) {
   extern __shared__ uint4 smem[];
   constexpr int G = FMT == ARCQ_FMT_NVFP4 ? 16 : 32;
   const int K = p.K, S = p.S, Kp = K + S;
   uint16_t *row = reinterpret_cast<uint16_t *>(smem);
   double *red = reinterpret_cast<double *>(row + K);  // one partial sum per wave
-  const int tid = threadIdx.x;
+  const int nwaves = (blockDim.x + 63) >> 6;
+  // Thread -> unit mapping rotated by whole waves per workgroup.  The waves that own the last
+  // select_num channels also encode the residual; a workgroup's wave i always lands on SIMD i, so
+  // without the rotation one SIMD of every CU would carry all of that extra work.
+  int tid = threadIdx.x + 64 * (int)(blockIdx.x % (unsigned)nwaves);
+  if (tid >= (int)blockDim.x) tid -= blockDim.x;
   const int nunits = K >> 4;                           // == number of working threads
   const bool active = tid < nunits;
   const int tail0 = (K - S) >> 4;
-  const int nwaves = (blockDim.x + 63) >> 6;
   const bool k_pow2 = (K & (K - 1)) == 0;
-  const double inv_k = 1.0 / (double)K;
+  const double inv_k = p.inv_k;
+  // SCALED: x32 = x / g (quantize.py:330) as q + (x - g*q)*rg with q = x*rg, rg = RN(1/g): the
+  // correctly rounded quotient for every bf16 x (checked exhaustively on the host).  A tensor scale
+  // outside 2^-60..2^60 in magnitude sends every unit through unit_exact.
+  const float g = SCALED ? (p.d_gscale ? *p.d_gscale : p.gscale) : 1.0f;
+  const float rg = SCALED ? 1.0f / g : 1.0f;
+  const bool g_odd = SCALED && !(fabsf(g) >= 0x1p-60f && fabsf(g) <= 0x1p+60f);
+  // a power-of-two tensor scale leaves bf16 operands bf16-valued: the coarse encode applies (and
+  // such operands sit on the grid's ties far too often for the two-sided test to pay)
+  const bool coarse = !SCALED || (f2u(g) & 0x7fffffu) == 0u;
+  // var + eps >= eps: with eps comfortably normal the square root needs no range scaling
+  const bool eps_normal = p.eps >= 0x1p-90f;
+
+  int r = blockIdx.x;
+  uint4 q0 = make_uint4(0, 0, 0, 0), q1 = q0;
+  if (r < p.rows && active) {  // first row in flight before anything that has to wait for memory
+    const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)r * K);
+    q0 = src[tid];
+    q1 = src[tid + nunits];
+  }
 
   // channel-only state, loaded once
   uint32_t addr[16];
@@ -299,13 +409,6 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
 #pragma unroll
   for (int i = 0; i < 16; ++i) yv[i] = 0u;  // low halves stay zero: only d16_hi loads write these
 
-  int r = blockIdx.x;
-  uint4 q0 = make_uint4(0, 0, 0, 0), q1 = q0;
-  if (r < p.rows && active) {
-    const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)r * K);
-    q0 = src[tid];
-    q1 = src[tid + nunits];
-  }
   for (; r < p.rows; r += gridDim.x) {
     uint4 n0 = q0, n1 = q1;
     if (r + (int)gridDim.x < p.rows && active) {  // prefetch the next row of this workgroup
@@ -328,11 +431,30 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
       ss = wave_sum_to_lane63(ss);
       if ((tid & 63) == 63) red[tid >> 6] = ss;
       lds_barrier();  // partial sums visible; the previous row's gathers are over
-      double tot = 0.0;
-      for (int w = 0; w < nwaves; ++w) tot += red[w];
+      double tot = 0.0, tot1 = 0.0;
+      int w = 0;
+      for (; w + 4 <= nwaves; w += 4) {  // two independent chains, 16-byte LDS reads
+        const double2 a = *reinterpret_cast<const double2 *>(red + w);
+        const double2 b = *reinterpret_cast<const double2 *>(red + w + 2);
+        tot += a.x;
+        tot1 += a.y;
+        tot += b.x;
+        tot1 += b.y;
+      }
+      for (; w < nwaves; ++w) tot += red[w];
+      tot += tot1;
       // mean = tot / K, exactly: a power-of-two K is a scaling, anything else an IEEE division
       const float var = k_pow2 ? (float)(tot * inv_k) : (float)(tot / (double)K);
-      const float rstd = 1.0f / sqrtf(var + p.eps);
+      const float a = var + p.eps;
+      float rstd;
+      if (eps_normal) {
+        // 1.0f / sqrtf(a) with both roundings, from the hardware estimates
+        const float sq = sqrt_from_estimate(a, __builtin_amdgcn_sqrtf(a));
+        rstd = rcp_from_estimate(sq, __builtin_amdgcn_rcpf(sq));
+        if (!(a < __builtin_inff())) rstd = a != a ? a : 0.0f;  // 1/sqrt(inf) = 0, NaN stays NaN
+      } else {
+        rstd = 1.0f / sqrtf(a);
+      }
       uint32_t yw[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -363,44 +485,73 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
 
     uint8_t *crow = p.codes + (size_t)r * (Kp >> 1);
     uint8_t *srow = p.scales + (size_t)r * (Kp / G);
+    if (SCALED) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) y[i] = div_bf16_by(y[i], g, rg);
+    }
     float s;
-    const uint32_t sb = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(div6_coarse(unit_amax3<FMT>(y)), &s)
-                                              : ue8m0_scale(div6_coarse(unit_amax3<FMT>(y)), &s);
-    const uint2 pk = encode_unit_coarse(y, scale_rcp<FMT>(s));
+    const float amax = unit_amax3<FMT>(y);
+    const float t = div6_any(amax);
+    uint32_t sb = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t, &s) : ue8m0_scale(t, &s);
+    uint2 pk;
+    bool redo = false;  // SCALED only: this unit needs unit_exact
+    if (coarse) {
+      pk = encode_unit_coarse(y, scale_rcp<FMT>(s));
+      if (SCALED) redo = amax_needs_exact(amax) || g_odd;
+    } else {
+      pk = encode_unit_two_sided(y, s, scale_rcp<FMT>(s));
+      redo = amax_needs_exact(amax) || g_odd;
+    }
+    const bool tail = active && tid >= tail0;
+    uint2 pk2 = pk;
+    uint32_t sb2 = sb;
+    if (MODE != MODE_W && tail) {
+      float e[16];
+      decode_unit(pk, e);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) e[i] = __builtin_fmaf(-e[i], s, y[i]);  // q*s is exact: the fp32 residual y - q*s
+      float s2;
+      const float amax2 = unit_amax3<FMT>(e);
+      const float t2 = div6_any(amax2);
+      sb2 = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t2, &s2) : ue8m0_scale(t2, &s2);
+      if (coarse) {
+        pk2 = encode_unit_coarse(e, scale_rcp<FMT>(s2));
+        if (SCALED) redo = amax_needs_exact(amax2) || redo;
+      } else {
+        pk2 = encode_unit_two_sided(e, s2, scale_rcp<FMT>(s2));
+        redo = amax_needs_exact(amax2) || redo;
+      }
+    }
+    if (SCALED && FMT == ARCQ_FMT_MXFP4) redo = __shfl_xor((int)redo, 1) != 0 || redo;  // both halves of a 32-block
+    if (SCALED && redo && active) {
+      if (MODE != MODE_W && tail) {
+        unit_exact<FMT, true>(yv, g, &pk, &sb, &pk2, &sb2);
+      } else {
+        unit_exact<FMT, false>(yv, g, &pk, &sb, &pk2, &sb2);
+        pk2 = pk;
+        sb2 = sb;
+      }
+    }
     if (active) {
       store_unit<FMT>(crow, srow, tid, pk, sb);
-      if (tid >= tail0) {
-        if (MODE == MODE_W) {
-          store_unit<FMT>(crow, srow, nunits + (tid - tail0), pk, sb);
-        } else {
-          float e[16];
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const uint32_t c = ((i < 8 ? pk.x : pk.y) >> (4 * (i & 7))) & 15u;
-            e[i] = y[i] - e2m1_value(c) * s;  // exact product, one rounding: the fp32 residual
-          }
-          float s2;
-          const uint32_t sb2 = block_scale<FMT>(unit_amax3<FMT>(e), &s2);
-          const uint2 pk2 = encode_unit_coarse(e, scale_rcp<FMT>(s2));
-          store_unit<FMT>(crow, srow, nunits + (tid - tail0), pk2, sb2);
-        }
-      }
+      if (tail) store_unit<FMT>(crow, srow, nunits + (tid - tail0), pk2, sb2);
     }
     q0 = n0;
     q1 = n1;
   }
 }
 
-template <int FMT, int MODE>
+template <int FMT, int MODE, bool SCALED>
 int launch_quantize_unit(const QuantParams &p, hipStream_t stream) {
   const int threads = (((p.K >> 4) + 63) / 64) * 64;
   const size_t lds = (size_t)p.K * 2 + 16 * sizeof(double);
   const int waves_per_wg = threads / 64;
-  // ~32 waves per CU resident at most; leave every workgroup a few rows to amortise its set-up
-  int grid = 256 * (32 / waves_per_wg > 0 ? 32 / waves_per_wg : 1);
+  // the kernel's register count lets 4 waves per SIMD (16 per CU) be resident: launch exactly the
+  // resident workgroups so that each amortises its set-up over as many rows as possible
+  int grid = 256 * (16 / waves_per_wg > 0 ? 16 / waves_per_wg : 1);
   if (const char *e = getenv("ARCQ_QUANT_GRID")) grid = atoi(e);
   if (grid > p.rows) grid = p.rows;
-  hipLaunchKernelGGL((quantize_rows_unit_kernel<FMT, MODE>), dim3(grid), dim3(threads), lds, stream, p);
+  hipLaunchKernelGGL((quantize_rows_unit_kernel<FMT, MODE, SCALED>), dim3(grid), dim3(threads), lds, stream, p);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }
@@ -491,17 +642,27 @@ int quantize_entry(int mode, const void *x, const void *gamma, float eps, int ro
   p.rows = rows;
   p.K = K;
   p.S = S;
+  p.inv_k = 1.0 / (double)K;
   hipStream_t st = static_cast<hipStream_t>(stream);
   // tensor scale known on the host to be 1: operands are exactly bf16 -> fast kernels
   if (!d_gscale && gscale == 1.0f && K <= 16384) {
     if (fmt == ARCQ_FMT_NVFP4) {
-      if (mode == MODE_X) return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_X>(p, st);
-      if (mode == MODE_W) return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_W>(p, st);
-      return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_NORM>(p, st);
+      if (mode == MODE_X) return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_X, false>(p, st);
+      if (mode == MODE_W) return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_W, false>(p, st);
+      return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_NORM, false>(p, st);
     }
-    if (mode == MODE_X) return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_X>(p, st);
-    if (mode == MODE_W) return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_W>(p, st);
-    return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_NORM>(p, st);
+    if (mode == MODE_X) return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_X, false>(p, st);
+    if (mode == MODE_W) return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_W, false>(p, st);
+    return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_NORM, false>(p, st);
+  }
+  // any other tensor scale, on the host or on the device: same kernel with the two-sided encode
+  if (mode != MODE_NORM && K <= 16384 && !getenv("ARCQ_QUANT_GENERIC")) {
+    if (fmt == ARCQ_FMT_NVFP4) {
+      if (mode == MODE_X) return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_X, true>(p, st);
+      return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_W, true>(p, st);
+    }
+    if (mode == MODE_X) return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_X, true>(p, st);
+    return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_W, true>(p, st);
   }
   if (fmt == ARCQ_FMT_NVFP4) {
     if (mode == MODE_X) return launch_quantize<ARCQ_FMT_NVFP4, MODE_X>(p, st);

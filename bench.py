@@ -219,7 +219,8 @@ def main():
 
     # ---------------- other quantize configurations (reported, not the headline) ----------------
     others = {}
-    gs_dev = torch.tensor(0.0625, device="cuda")
+    # the NVFP4 tensor scale the reference's callers compute: max|x| / (448 * 6) (model/qLlamaLayer.py:74)
+    gs_dev = (xs[0].abs().max().float() / 2688.0).reshape(())
     for fmt, S, kind in (("MXFP4", 256, "norm"), ("NVFP4", 64, "norm"), ("NVFP4", 256, "x_unit"), ("MXFP4", 256, "x_unit"),
                          ("NVFP4", 256, "x_scaled")):
         q, sf = outputs(fmt, S)

@@ -98,3 +98,40 @@ def test_coarse_fast_encode_is_exact(hm, fmt, residual):
 
 def test_div6_coarse_is_exact(hm):
     assert hm.arcq_host_check_div6() == 0
+
+
+def test_div6_any_is_exact(hm):
+    """a/6 as three fused operations equals the IEEE quotient for every fp32 significand"""
+    hm.arcq_host_check_div6_any.restype = ctypes.c_long
+    assert hm.arcq_host_check_div6_any() == 0
+
+
+def test_bf16_by_tensor_scale_division_is_exact(hm):
+    """x/g (model/quantize.py:330) as q + (x - g*q)*rg for every bf16 significand of x and every
+    fp32 significand of g, both signs"""
+    hm.arcq_host_check_div_bf16.restype = ctypes.c_long
+    hm.arcq_host_check_div_bf16.argtypes = [ctypes.c_int]
+    assert hm.arcq_host_check_div_bf16(1) == 0
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_two_sided_encode_is_exact(hm, fmt):
+    """the encode used for tensor scales != 1 (two hardware conversions; e2m1_resolve where they
+    differ) gives the reference's code for random operands and for +-200 ulp around every decision
+    point, every scale, reciprocal off by -1/0/+1 ulp; the two conversions agree almost always"""
+    hm.arcq_host_check_two_sided.restype = ctypes.c_longlong
+    hm.arcq_host_check_two_sided.argtypes = [ctypes.c_int, ctypes.c_long, ctypes.POINTER(ctypes.c_longlong),
+                                             ctypes.POINTER(ctypes.c_longlong)]
+    acc, cnt = ctypes.c_longlong(), ctypes.c_longlong()
+    bad = hm.arcq_host_check_two_sided(fmt, 500_000, ctypes.byref(acc), ctypes.byref(cnt))
+    assert bad == 0
+    assert cnt.value > 50_000_000
+    assert acc.value / cnt.value > 0.999
+
+
+def test_rstd_from_hardware_estimates_is_exact(hm):
+    """1/sqrt(var + eps) of the fused RMSNorm kernel: sqrt and reciprocal rebuilt from 1-ulp estimates
+    equal 1.0f / sqrtf(a) (two roundings) on a dense stretch of fp32 and across the exponent range"""
+    hm.arcq_host_check_rstd.restype = ctypes.c_long
+    hm.arcq_host_check_rstd.argtypes = [ctypes.c_long]
+    assert hm.arcq_host_check_rstd(40_000_000) == 0
