@@ -677,6 +677,194 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
                                wave, lane);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Skinny kernels for M <= 64 (decode batches): the GEMM is a stream of the weight matrix, read
+// exactly once, so nothing is staged through LDS.  A workgroup owns 16 weight rows; its four waves
+// take the K steps of 128 round-robin in pairs (split-K: wave w does steps 2w, 2w+1, 2w+8, 2w+9, ...:
+// a pair of steps is one whole 128-byte line of every row, and the four waves walk neighbouring lines) and their partial sums meet in LDS.  A lane loads
+// the 16 bytes (32 codes) the 16x16 MFMA wants from it straight from global memory: row lane%16,
+// K group lane/16, i.e. 64 contiguous bytes per row and step.  The activations (<= 64 rows) come
+// from L2 the same way, one 16-column tile at a time, each reusing the weight registers.
+// Requires K' % 128 == 0 and 16-byte aligned scale arrays.
+// ---------------------------------------------------------------------------------------------
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int MT, int AT>
+__device__ __forceinline__ void skinny_reduce_store(const GemmParams &p, v4f (&acc)[AT * MT], float (*red)[MT * AT][64][4],
+                                                    int wave, int lane) {
+  if (wave > 0) {
+#pragma unroll
+    for (int j = 0; j < AT * MT; ++j) *reinterpret_cast<v4f *>(red[wave - 1][j][lane]) = acc[j];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  const float alpha = effective_alpha(p);
+#pragma unroll
+  for (int i = 0; i < AT; ++i) {
+    const int n0 = ((int)blockIdx.x * AT + i) * 16 + 4 * (lane >> 4);
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      v4f t = acc[i * MT + j];
+#pragma unroll
+      for (int w = 0; w < 3; ++w) t += *reinterpret_cast<const v4f *>(red[w][i * MT + j][lane]);
+      const int m = 16 * j + (lane & 15);
+      if (m >= p.M) continue;
+      uint16_t *dst = p.c + (size_t)m * p.N + n0;
+      if (n0 + 3 < p.N && (p.N & 3) == 0) {
+        const uint32_t lo = f32_to_bf16_bits(t[0] * alpha) | (f32_to_bf16_bits(t[1] * alpha) << 16);
+        const uint32_t hi = f32_to_bf16_bits(t[2] * alpha) | (f32_to_bf16_bits(t[3] * alpha) << 16);
+        *reinterpret_cast<uint2 *>(dst) = make_uint2(lo, hi);
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (n0 + v < p.N) dst[v] = (uint16_t)f32_to_bf16_bits(t[v] * alpha);
+      }
+    }
+  }
+}
+
+template <int MT, int AT>
+__global__ __launch_bounds__(256) void gemm_mxfp4_skinny(GemmParams p) {
+  __shared__ float red[3][MT * AT][64][4];
+  constexpr int D = (MT * AT >= 4) ? 4 : 8;  // K steps whose loads are in flight together
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int T = p.Kp >> 7;
+  const size_t rowb = (size_t)(p.Kp >> 1), rows = (size_t)(p.Kp >> 5);
+  const uint8_t *wc[AT], *ws[AT], *xc[MT], *xs[MT];
+#pragma unroll
+  for (int i = 0; i < AT; ++i) {
+    const int n = min(((int)blockIdx.x * AT + i) * 16 + r, p.N - 1);
+    wc[i] = p.b_codes + n * rowb + 16 * g;
+    ws[i] = p.b_scales + n * rows;
+  }
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int m = min(16 * j + r, p.M - 1);
+    xc[j] = p.a_codes + m * rowb + 16 * g;
+    xs[j] = p.a_scales + m * rows;
+  }
+  v4f acc[AT * MT];
+#pragma unroll
+  for (int j = 0; j < AT * MT; ++j) acc[j] = v4f{0.f, 0.f, 0.f, 0.f};
+  const uint32_t sh = 8u * (uint32_t)g;
+  for (int t0 = 2 * wave; t0 < T; t0 += 4 * D) {
+    uint4 a[AT][D], b[MT][D];
+    uint32_t sa[AT][D], sb[MT][D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int t = t0 + 8 * (d >> 1) + (d & 1);
+      if (t < T) {  // uniform over the wave
+#pragma unroll
+        for (int i = 0; i < AT; ++i) {
+          a[i][d] = *reinterpret_cast<const uint4 *>(wc[i] + 64 * t);
+          sa[i][d] = *reinterpret_cast<const uint32_t *>(ws[i] + 4 * t);
+        }
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          b[j][d] = *reinterpret_cast<const uint4 *>(xc[j] + 64 * t);
+          sb[j][d] = *reinterpret_cast<const uint32_t *>(xs[j] + 4 * t);
+        }
+      }
+    }
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      if (t0 + 8 * (d >> 1) + (d & 1) < T) {
+#pragma unroll
+        for (int i = 0; i < AT; ++i)
+#pragma unroll
+          for (int j = 0; j < MT; ++j)
+            acc[i * MT + j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                fp4_operand(a[i][d]), fp4_operand(b[j][d]), acc[i * MT + j], 4, 4, 0, (int)(sa[i][d] >> sh), 0,
+                (int)(sb[j][d] >> sh));
+      }
+    }
+  }
+  skinny_reduce_store<MT, AT>(p, acc, red, wave, lane);
+}
+
+// NVFP4: the same walk; a lane's 16 bytes are two blocks of 16, decoded to fp16 eight codes at a
+// time and fed to four v_mfma_f32_16x16x32_f16.  Which K index a lane supplies to which of the four
+// is free as long as both operands agree: here MFMA d of a step takes K = 128t + 32*(lane/16) + 8d..+7.
+template <int MT>
+__global__ __launch_bounds__(256) void gemm_nvfp4_skinny(GemmParams p) {
+  __shared__ float red[3][MT][64][4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int T = p.Kp >> 7;
+  const size_t rowb = (size_t)(p.Kp >> 1), rows = (size_t)(p.Kp >> 4);
+  const int n = min((int)blockIdx.x * 16 + r, p.N - 1);
+  const uint8_t *wc = p.b_codes + n * rowb + 16 * g;
+  const uint8_t *ws = p.b_scales + n * rows + 2 * g;
+  const uint8_t *xc[MT], *xs[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int m = min(16 * j + r, p.M - 1);
+    xc[j] = p.a_codes + m * rowb + 16 * g;
+    xs[j] = p.a_scales + m * rows + 2 * g;
+  }
+  v4f acc[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) acc[j] = v4f{0.f, 0.f, 0.f, 0.f};
+  constexpr int D = MT >= 4 ? 2 : 4;  // K steps whose loads are in flight together
+  for (int t0 = 2 * wave; t0 < T; t0 += 4 * D) {
+    uint4 aq[D], bq[MT][D];
+    uint32_t as2[D], bs2[MT][D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int t = t0 + 8 * (d >> 1) + (d & 1);
+      if (t < T) {  // uniform over the wave
+        aq[d] = *reinterpret_cast<const uint4 *>(wc + 64 * t);
+        as2[d] = *reinterpret_cast<const uint16_t *>(ws + 8 * t);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          bq[j][d] = *reinterpret_cast<const uint4 *>(xc[j] + 64 * t);
+          bs2[j][d] = *reinterpret_cast<const uint16_t *>(xs[j] + 8 * t);
+        }
+      }
+    }
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      if (t0 + 8 * (d >> 1) + (d & 1) < T) {
+        const uint32_t ap = nv_scale_pair_f16((as2[d] & 0xffu) | ((as2[d] & 0xff00u) << 8));
+        const v8h a0 = decode8_nvfp4_f16<false>(aq[d].x, ap), a1 = decode8_nvfp4_f16<false>(aq[d].y, ap);
+        const v8h a2 = decode8_nvfp4_f16<true>(aq[d].z, ap), a3 = decode8_nvfp4_f16<true>(aq[d].w, ap);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          const uint32_t bp = nv_scale_pair_f16((bs2[j][d] & 0xffu) | ((bs2[j][d] & 0xff00u) << 8));
+          const uint4 q = bq[j][d];
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, decode8_nvfp4_f16<false>(q.x, bp), acc[j], 0, 0, 0);
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, decode8_nvfp4_f16<false>(q.y, bp), acc[j], 0, 0, 0);
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a2, decode8_nvfp4_f16<true>(q.z, bp), acc[j], 0, 0, 0);
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a3, decode8_nvfp4_f16<true>(q.w, bp), acc[j], 0, 0, 0);
+        }
+      }
+    }
+  }
+  skinny_reduce_store<MT, 1>(p, acc, red, wave, lane);
+}
+
+template <int FMT, int MT, int AT>
+int launch_skinny(const GemmParams &p, hipStream_t st) {
+  const int grid = (p.N + 16 * AT - 1) / (16 * AT);
+  if (FMT == ARCQ_FMT_MXFP4)
+    hipLaunchKernelGGL((gemm_mxfp4_skinny<MT, AT>), dim3(grid), dim3(256), 0, st, p);
+  else
+    hipLaunchKernelGGL((gemm_nvfp4_skinny<MT>), dim3(grid), dim3(256), 0, st, p);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+template <int FMT>
+int launch_skinny_for(const GemmParams &p, hipStream_t st) {
+  // two 16-row weight tiles per wave (halving the activation reads) measured no better: experiments only
+  static const int at_env = getenv("ARCQ_GEMM_SKINNY_AT") ? atoi(getenv("ARCQ_GEMM_SKINNY_AT")) : 0;
+  const bool at2 = FMT == ARCQ_FMT_MXFP4 && at_env == 2;
+  if (p.M <= 16) return at2 ? launch_skinny<FMT, 1, 2>(p, st) : launch_skinny<FMT, 1, 1>(p, st);
+  if (p.M <= 32) return at2 ? launch_skinny<FMT, 2, 2>(p, st) : launch_skinny<FMT, 2, 1>(p, st);
+  return launch_skinny<FMT, 4, 1>(p, st);
+}
+
 template <int WN, int WM>
 int launch_nvfp4_tiled(const GemmParams &p, hipStream_t st) {
   constexpr int BN = 64 * WN, BM = 64 * WM;
@@ -727,14 +915,24 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
   // few rows of activations -> small tiles so that enough workgroups exist; many -> large tiles
   // for operand reuse.  K' % 128 != 0 goes to the direct kernels.
   static const int force = getenv("ARCQ_GEMM_KERNEL") ? atoi(getenv("ARCQ_GEMM_KERNEL")) : -1;
-  if (fmt == ARCQ_FMT_MXFP4 && force != 0 && Kp % 128 == 0) {
+  static const int skinny_max = getenv("ARCQ_GEMM_SKINNY_MAX") ? atoi(getenv("ARCQ_GEMM_SKINNY_MAX")) : 64;
+  const bool fast_ok = Kp % 128 == 0 && aligned16(a_scales) && aligned16(b_scales);
+  // Measured crossover against the tiled kernels (weights streaming from HBM): the skinny kernels
+  // re-read the activations from L2 once per 16 weight rows, which costs more the larger M and N are.
+  const bool skinny_wins = fmt == ARCQ_FMT_MXFP4
+                               ? (N <= 4096 || (N <= 8192 && (M <= 32 || Kp >= 8192)) || M <= 4)
+                               : (N <= 8192 || M <= 16);
+  if (fast_ok && (force == 1 || (force < 0 && M <= skinny_max && skinny_wins)) && M <= 64) {
+    return fmt == ARCQ_FMT_MXFP4 ? launch_skinny_for<ARCQ_FMT_MXFP4>(p, st) : launch_skinny_for<ARCQ_FMT_NVFP4>(p, st);
+  }
+  if (fmt == ARCQ_FMT_MXFP4 && force != 0 && fast_ok) {
     if (force == 44) return launch_mxfp4_tiled<4, 4>(p, st);
     if (force == 42 || (force < 0 && M > 1024)) return launch_mxfp4_tiled<4, 2>(p, st);
     if (force == 24) return launch_mxfp4_tiled<2, 4>(p, st);
     if (force == 22 || (force < 0 && M > 128)) return launch_mxfp4_tiled<2, 2>(p, st);
     if (force == 21 || force < 0) return launch_mxfp4_tiled<2, 1>(p, st);
   }
-  if (fmt == ARCQ_FMT_NVFP4 && force != 0 && Kp % 128 == 0) {
+  if (fmt == ARCQ_FMT_NVFP4 && force != 0 && fast_ok) {
     if (force == 44 || (force < 0 && M > 1024)) return launch_nvfp4_tiled<4, 4>(p, st);
     if (force == 42) return launch_nvfp4_tiled<4, 2>(p, st);
     if (force == 22 || (force < 0 && M > 128)) return launch_nvfp4_tiled<2, 2>(p, st);

@@ -96,36 +96,62 @@ def cpu_baseline(torch, sample_rows):
                       f"model/quantize.py fake_reorder_quantize_x after HF RMSNorm), best of {runs} runs, {best:.3f} s each"}
 
 
-def gemm_rows(torch, agemm, shapes, Ms, fmts, iters=20):
+def gemm_rows(torch, agemm, shapes, Ms, fmts, iters=40):
+    """ARC GEMM through the C ABI on preallocated outputs.  The quantized weights rotate over enough
+    copies (> 300 MB) that every launch streams them from HBM, as a model's layers do; the bf16
+    comparison rotates the same way.  For M <= 64 the bound is the weight stream, reported as GB/s."""
+    import ctypes
     import recipes
+    from arcquant_amd import _lib
+    L = _lib.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    fid = {"NVFP4": 0, "MXFP4": 1}
     rows = []
     for (N, K) in shapes:
         S = 256
         Kp = K + S
         w = recipes.weights(N, K, seed=3).cuda()
         idx = torch.arange(K, dtype=torch.int16, device="cuda")
-        wq = {f: agemm.reorder_quantize_w(w, idx, S, fmt=f, global_scale=recipes.tensor_scale(w.cpu(), f)) for f in fmts}
+        wq = {}
+        for f in fmts:
+            b, sfb = agemm.reorder_quantize_w(w, idx, S, fmt=f, global_scale=recipes.tensor_scale(w.cpu(), f))
+            ncopy = max(2, int(3.2e8 // (b.numel() + sfb.numel())) + 1)
+            wq[f] = [(b.clone(), sfb.clone()) for _ in range(ncopy)]
+        nb = max(2, int(3.2e8 // (N * Kp * 2)) + 1)
+        wbs = [torch.randn(N, Kp, device="cuda", dtype=torch.bfloat16) for _ in range(nb)]
         for M in Ms:
             x = recipes.activations(M, K, seed=1).cuda()
             row = {"N": N, "K": K, "Kp": Kp, "M": M}
+            c = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
             for f in fmts:
                 a, sfa = agemm.reorder_quantize_x(x, idx, S, fmt=f, global_scale=recipes.tensor_scale(x.cpu(), f))
-                b, sfb = wq[f]
-                fn = lambda i: agemm.matmul(a, b, sfa, sfb, 1.0, fmt=f)
-                for i in range(3):
+                ws = wq[f]
+
+                def fn(i, a=a, sfa=sfa, ws=ws, f=f):
+                    b, sfb = ws[i % len(ws)]
+                    L.arcq_matmul(a.data_ptr(), sfa.data_ptr(), b.data_ptr(), sfb.data_ptr(), M, N, Kp, fid[f], 1.0,
+                                  None, None, c.data_ptr(), stream)
+                for i in range(5):
                     fn(i)
                 ms = loop_time_ms(fn, iters, torch)
-                row[f] = {"ms": round(ms, 4), "tflops": round(gemm_flops(M, N, Kp) / ms / 1e9, 1),
+                row[f] = {"us": round(ms * 1e3, 2), "tflops": round(gemm_flops(M, N, Kp) / ms / 1e9, 1),
                           "frac_of_mfma_peak": round(gemm_flops(M, N, Kp) / ms / 1e9 / MFMA_PEAK_TFLOPS[f], 4)}
+                if M <= 64:
+                    wbytes = ws[0][0].numel() + ws[0][1].numel()
+                    row[f]["weight_stream_GB/s"] = round(wbytes / ms / 1e6, 1)
+                    row[f]["frac_hbm"] = round(wbytes / ms / 1e6 / HBM_PEAK_GBS, 4)
             xa = torch.randn(M, Kp, device="cuda", dtype=torch.bfloat16)
-            wb = torch.randn(N, Kp, device="cuda", dtype=torch.bfloat16)
-            fn = lambda i: torch.matmul(xa, wb.t())
-            for i in range(3):
+            fn = lambda i: torch.matmul(xa, wbs[i % nb].t(), out=c)
+            for i in range(5):
                 fn(i)
             ms = loop_time_ms(fn, iters, torch)
-            row["bf16_torch"] = {"ms": round(ms, 4), "tflops": round(gemm_flops(M, N, Kp) / ms / 1e9, 1)}
+            row["bf16_torch"] = {"us": round(ms * 1e3, 2), "tflops": round(gemm_flops(M, N, Kp) / ms / 1e9, 1)}
+            for f in fmts:
+                row[f]["vs_bf16"] = round(row["bf16_torch"]["us"] / row[f]["us"], 2)
             rows.append(row)
             print("[bench] gemm", json.dumps(row), file=sys.stderr, flush=True)
+        del wq, wbs
+        torch.cuda.empty_cache()
     return rows
 
 
@@ -257,7 +283,7 @@ def main():
 
     if not args.no_gemm:
         shapes = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)] if args.gemm_table else [(6144, 4096)]
-        Ms = [1, 16, 128, 512, 2048, 4096] if args.gemm_table else [16, 512, 4096]
+        Ms = [1, 16, 64, 128, 512, 2048, 4096] if args.gemm_table else [1, 16, 512, 4096]
         out["gemm"] = gemm_rows(torch, agemm, shapes, Ms, ["MXFP4", "NVFP4"])
         out["gemm_peaks_tflops"] = MFMA_PEAK_TFLOPS
 

@@ -109,3 +109,29 @@ def test_matmul_llama_shapes_vs_torch_fp32(agemm, fmt, M, N, K, S):
     # and the whole scheme tracks the unquantized product
     y_true = x.cuda().float() @ w.cuda().float().T
     assert rel_fro(y.float(), y_true) < 0.2
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 32, 48, 64])
+@pytest.mark.parametrize("N,K,S", [(6144, 4096, 256), (202, 384, 0), (4100, 1024, 128)])
+def test_matmul_decode_batches(agemm, fmt, M, N, K, S):
+    """M <= 64 (decode batches) at a benchmark shape and at shapes whose N is not a multiple of the
+    16-row strips or of the 4-wide stores: against torch's fp32 matmul of the dequantized operands,
+    and, row by row, against the same call on a 128-row batch that contains these rows (another
+    kernel computes that one)."""
+    (x, w, idx, gx, gw), (a, sfa, b, sfb) = quantized_pair(agemm, 128, N, K, S, fmt, seed=11)
+    print(f"matmul decode {fmt} M={M} N={N} K={K} S={S}", flush=True)
+    a_m = a[:M].contiguous()
+    sfa_m = sfa.view(128, -1)[:M].contiguous().view(-1)
+    y = agemm.matmul(a_m, b, sfa_m, sfb, gx * gw)
+    assert y.shape == (M, N)
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        want = (agemm.dequantize(a_m, sfa_m, fmt=fmt) @ agemm.dequantize(b, sfb, fmt=fmt).T) * (gx * gw)
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    assert rel_fro(y.float(), want) < TOL
+    y_big = agemm.matmul(a, b, sfa, sfb, gx * gw)[:M]
+    # same operands, fp32 accumulation in another order, one bf16 rounding each
+    assert rel_fro(y.float(), y_big.float()) < 4e-3
