@@ -1,0 +1,329 @@
+"""Layer-level callers of the ARC hot path: counterparts of the reference's Python layer code,
+built on arcquant_amd.agemm (libarcq_hip.so) and nothing else.
+
+    reorder_quantize_x      model/qLlamaLayer.py:73-86     (activation quantizer + NVFP4 tensor scale)
+    QLinearLayer            model/qLinearLayer.py:30-81    (quantized weights, forward on the tuple)
+    RMSNormQuant            benchmarks/modeling_arc.py:211-227 (fused RMSNorm -> quantize)
+    LlamaMLP / LlamaAttention / LlamaDecoderLayer
+                            model/qLlamaLayer.py:281-443, benchmarks/modeling_arc.py:80-330
+    MixtralSparseMoeBlock   model/qMixtralLayer.py:388-543
+
+The protocol between a quantizer and the linears that consume it is the reference's tuple
+``(qx, scale_x, scale, bsz, q_len)`` (model/qLinearLayer.py:66): packed codes, block-scale bytes,
+tensor scale, and the shape to restore.
+
+What differs from the reference, on purpose:
+  * nothing synchronises with the host.  The reference calls torch.cuda.synchronize() after every
+    quantizer and every GEMM (model/qLlamaLayer.py:298, model/qLinearLayer.py:73) and turns the
+    tensor scales into python floats (an implicit .item()); here the NVFP4 tensor scales stay
+    0-dim device tensors that the kernels read themselves.
+  * x / scale is done inside the quantizer in fp32 (model/quantize.py:330), not in bf16 before it
+    (model/qLlamaLayer.py:76).
+  * quant_type 'MXFP4' runs the real kernels too; the reference falls back to fake-quantized bf16
+    tensors and F.linear for it (model/qLinearLayer.py:71).
+  * the MoE block sorts tokens by expert on the device and reads the eight counts back once,
+    instead of one torch.where (a host sync) per expert.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import agemm
+
+NVFP4_RANGE = 448.0 * 6.0   # model/qLlamaLayer.py:74
+
+
+def _tensor_scale(t: torch.Tensor, signed: bool) -> torch.Tensor:
+    """NVFP4 tensor scale as a 0-dim fp32 device tensor.  Activations: max|x| / 2688
+    (model/qLlamaLayer.py:74); weights: the signed max (model/qLinearLayer.py:26).  A zero tensor
+    gets scale 1 (the reference would divide by zero)."""
+    m = (t.max() if signed else t.abs().max()).float()
+    # tensor / tensor: an IEEE division.  Dividing by a python number would make torch multiply by
+    # the rounded reciprocal on the GPU, one ulp away from the CPU result for many inputs.
+    m = m / torch.full_like(m, NVFP4_RANGE)
+    return torch.where(m == 0, torch.ones_like(m), m)
+
+
+def reorder_quantize_x(x, reorder_index, select_num, quant_type="NVFP4"):
+    """model/qLlamaLayer.py:79-86: x bf16 [tokens, K] -> (qx, scale_x, scale)."""
+    if quant_type == "NVFP4":
+        scale = _tensor_scale(x, signed=False)
+        qx, scale_x = agemm.reorder_quantize_x(x, reorder_index, select_num, fmt="NVFP4", global_scale=scale)
+        return qx, scale_x, scale
+    qx, scale_x = agemm.reorder_quantize_x(x, reorder_index, select_num, fmt=quant_type)
+    return qx, scale_x, 1.0
+
+
+def quantize_tokens(hidden_states, reorder_index, select_num, quant_type="NVFP4"):
+    """[bsz, q_len, K] or [tokens, K] -> the 5-tuple a QLinearLayer takes."""
+    if hidden_states.dim() == 3:
+        bsz, q_len, _ = hidden_states.shape
+        flat = hidden_states.reshape(bsz * q_len, -1)
+    else:
+        bsz, q_len = None, hidden_states.shape[0]
+        flat = hidden_states
+    qx, sfx, scale = reorder_quantize_x(flat.contiguous(), reorder_index, select_num, quant_type)
+    return qx, sfx, scale, bsz, q_len
+
+
+class QLinearLayer(nn.Module):
+    """model/qLinearLayer.py:30-81.  Weights are quantized once at construction with the input
+    channels reordered by `reorder_index` and the last `select_num` of them repeated."""
+
+    def __init__(self, originalLayer: nn.Linear, select_num, reorder_index, out_reorder_index=None,
+                 quant_type="NVFP4"):
+        super().__init__()
+        self.in_features = originalLayer.in_features
+        self.out_features = originalLayer.out_features
+        self.select_num = int(select_num)
+        self.quant_type = quant_type
+        w = originalLayer.weight.data
+        if not w.is_cuda:
+            raise RuntimeError("QLinearLayer quantizes on the GPU: move the layer to a cuda device first")
+        w = w.to(torch.bfloat16).contiguous()
+        idx = reorder_index.to(device=w.device, dtype=torch.int16).contiguous()
+        if quant_type == "NVFP4":
+            scale = _tensor_scale(w, signed=True)
+            W, scale_w = agemm.reorder_quantize_w(w, idx, self.select_num, fmt="NVFP4", global_scale=scale)
+        else:
+            scale = torch.ones((), dtype=torch.float32, device=w.device)
+            W, scale_w = agemm.reorder_quantize_w(w, idx, self.select_num, fmt=quant_type)
+        self.register_buffer("W", W)
+        self.register_buffer("scale_w", scale_w)
+        self.register_buffer("scale", scale)
+        if originalLayer.bias is not None:
+            self.register_buffer("bias", originalLayer.bias.data.to(torch.bfloat16))
+        else:
+            self.bias = None
+
+    @torch.no_grad()
+    def forward(self, x):
+        qx, scale_x, scale, bsz, q_len = x
+        alpha = (scale, self.scale) if isinstance(scale, torch.Tensor) else (float(scale), self.scale)
+        y = agemm.matmul(qx, self.W, scale_x, self.scale_w, alpha, fmt=self.quant_type)
+        if self.bias is not None:
+            y = y + self.bias
+        if bsz is not None:
+            return y.reshape(bsz, q_len, -1)
+        return y.reshape(q_len, -1)
+
+
+class RMSNormQuant(nn.Module):
+    """benchmarks/modeling_arc.py:211-227: RMSNorm fused with the activation quantizer; returns the
+    tuple directly (tensor scale 1, as the reference's op has none)."""
+
+    def __init__(self, weight, eps, select_num, reorder_index, quant_type="NVFP4"):
+        super().__init__()
+        self.register_buffer("weight", weight.to(torch.bfloat16).contiguous())
+        self.register_buffer("reorder_index", reorder_index.to(torch.int16).contiguous())
+        self.variance_epsilon = float(eps)
+        self.select_num = int(select_num)
+        self.quant_type = quant_type
+
+    @torch.no_grad()
+    def forward(self, hidden_states):
+        bsz, q_len, _ = hidden_states.shape
+        flat = hidden_states.reshape(bsz * q_len, -1).contiguous()
+        A, SFA = agemm.rmsnorm_quantize_x(flat, self.weight, self.variance_epsilon, self.reorder_index,
+                                          self.select_num, fmt=self.quant_type)
+        return A, SFA, 1.0, bsz, q_len
+
+
+def _rotate_half(x):
+    h = x.shape[-1] // 2
+    return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+
+
+def rotary_pos_emb(q, k, beg, base=10000.0):
+    """benchmarks/modeling_arc.py:63-78: rotary embedding for positions beg .. beg+seqlen."""
+    dim, seqlen = q.shape[-1], q.shape[-2]
+    inv_freq = 1.0 / (base ** (torch.arange(0, dim, 2, device=q.device).float() / dim))
+    t = torch.arange(beg, beg + seqlen, device=q.device, dtype=torch.float32)
+    freqs = torch.outer(t, inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)[None, None]
+    cos, sin = emb.cos().to(q.dtype), emb.sin().to(q.dtype)
+    return q * cos + _rotate_half(q) * sin, k * cos + _rotate_half(k) * sin
+
+
+def _linear(out_features, in_features, std, device, gen):
+    lin = nn.Linear(in_features, out_features, bias=False, device=device, dtype=torch.bfloat16)
+    w = torch.randn(out_features, in_features, generator=gen) * std
+    lin.weight.data.copy_(w.to(torch.bfloat16))
+    return lin
+
+
+class LlamaMLP(nn.Module):
+    """SwiGLU MLP with gate and up projections fused into one [2*inter, hidden] linear
+    (model/qLlamaLayer.py:380-443 with the fusion of benchmark configuration 4)."""
+
+    def __init__(self, gate_up: nn.Linear, down: nn.Linear, select_num_in, select_num_down, in_index, down_index,
+                 quant_type="NVFP4"):
+        super().__init__()
+        self.inter = down.in_features
+        self.gate_up_proj = QLinearLayer(gate_up, select_num_in, in_index, quant_type=quant_type)
+        self.down_proj = QLinearLayer(down, select_num_down, down_index, quant_type=quant_type)
+        self.register_buffer("down_reorder_index", down_index.to(torch.int16))
+        self.quant_type = quant_type
+
+    @torch.no_grad()
+    def forward(self, x):
+        """x: the tuple of the already quantized (normalised) hidden states"""
+        gu = self.gate_up_proj(x)
+        t = F.silu(gu[..., :self.inter]) * gu[..., self.inter:]
+        return self.down_proj(quantize_tokens(t, self.down_reorder_index, self.down_proj.select_num, self.quant_type))
+
+
+class LlamaAttention(nn.Module):
+    """Grouped-query attention with a fused qkv projection, bf16 SDPA and a preallocated bf16 KV
+    cache (model/qLlamaLayer.py:207-378; the INT4 paged cache of model/kv_cache.py is a separate path)."""
+
+    def __init__(self, qkv: nn.Linear, o: nn.Linear, num_heads, num_kv_heads, select_num_in, select_num_o, in_index,
+                 o_index, quant_type="NVFP4"):
+        super().__init__()
+        self.num_heads, self.num_kv_heads = num_heads, num_kv_heads
+        self.head_dim = o.in_features // num_heads
+        self.qkv_proj = QLinearLayer(qkv, select_num_in, in_index, quant_type=quant_type)
+        self.o_proj = QLinearLayer(o, select_num_o, o_index, quant_type=quant_type)
+        self.register_buffer("o_reorder_index", o_index.to(torch.int16))
+        self.quant_type = quant_type
+
+    @torch.no_grad()
+    def forward(self, x, kv_cache=None, past_len=0):
+        """x: quantized hidden states (tuple).  kv_cache: None or (k, v) bf16 [bsz, kv_heads, L, d]
+        holding past_len valid positions; the new keys/values are written behind them."""
+        bsz, q_len = x[3], x[4]
+        d, nh, nkv = self.head_dim, self.num_heads, self.num_kv_heads
+        qkv = self.qkv_proj(x)
+        q = qkv[..., :nh * d].view(bsz, q_len, nh, d).transpose(1, 2)
+        k = qkv[..., nh * d:(nh + nkv) * d].view(bsz, q_len, nkv, d).transpose(1, 2)
+        v = qkv[..., (nh + nkv) * d:].view(bsz, q_len, nkv, d).transpose(1, 2)
+        q, k = rotary_pos_emb(q, k, past_len)
+        if kv_cache is not None:
+            kc, vc = kv_cache
+            kc[:, :, past_len:past_len + q_len] = k
+            vc[:, :, past_len:past_len + q_len] = v
+            k, v = kc[:, :, :past_len + q_len], vc[:, :, :past_len + q_len]
+        out = F.scaled_dot_product_attention(q, k, v, is_causal=(q_len > 1 and past_len == 0),
+                                             enable_gqa=(nkv != nh))
+        out = out.transpose(1, 2).reshape(bsz, q_len, nh * d)
+        return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num, self.quant_type))
+
+
+class LlamaDecoderLayer(nn.Module):
+    """One decoder layer: x + attn(norm_quant(x)), then + mlp(norm_quant(.)), with both RMSNorms
+    fused into the quantizer (benchmarks/modeling_arc.py:262-330)."""
+
+    def __init__(self, hidden, inter, num_heads, num_kv_heads, eps=1e-5, select_num=256, select_num_down=256,
+                 quant_type="NVFP4", indices=None, seed=4, device="cuda"):
+        super().__init__()
+        gen = torch.Generator().manual_seed(seed)
+        d = hidden // num_heads
+        ident = lambda n: torch.arange(n, dtype=torch.int16, device=device)
+        idx = indices or {}
+        in_attn = idx.get("attn_in", ident(hidden))
+        in_mlp = idx.get("mlp_in", ident(hidden))
+        o_idx = idx.get("o_in", ident(hidden))
+        down_idx = idx.get("down_in", ident(inter))
+        self.linears = {   # the bf16 originals, kept for comparisons; not registered, not used in forward
+            "qkv": _linear((num_heads + 2 * num_kv_heads) * d, hidden, 0.02, device, gen),
+            "o": _linear(hidden, hidden, 0.02, device, gen),
+            "gate_up": _linear(2 * inter, hidden, 0.02, device, gen),
+            "down": _linear(hidden, inter, 0.02, device, gen),
+        }
+        g1 = (torch.rand(hidden, generator=gen) + 0.5).to(torch.bfloat16).to(device)
+        g2 = (torch.rand(hidden, generator=gen) + 0.5).to(torch.bfloat16).to(device)
+        self.input_layernorm = RMSNormQuant(g1, eps, select_num, in_attn, quant_type)
+        self.post_attention_layernorm = RMSNormQuant(g2, eps, select_num, in_mlp, quant_type)
+        self.self_attn = LlamaAttention(self.linears["qkv"], self.linears["o"], num_heads, num_kv_heads, select_num,
+                                        select_num, in_attn, o_idx, quant_type)
+        self.mlp = LlamaMLP(self.linears["gate_up"], self.linears["down"], select_num, select_num_down, in_mlp,
+                            down_idx, quant_type)
+
+    @torch.no_grad()
+    def forward(self, hidden_states, kv_cache=None, past_len=0):
+        h = hidden_states + self.self_attn(self.input_layernorm(hidden_states), kv_cache, past_len)
+        return h + self.mlp(self.post_attention_layernorm(h))
+
+
+class MixtralExpertMLP(nn.Module):
+    """model/qMixtralLayer.py:466-543: w2(act(w1 x) * w3 x) on a ragged set of tokens."""
+
+    def __init__(self, w1: nn.Linear, w3: nn.Linear, w2: nn.Linear, select_num, in_index, w2_index, quant_type="NVFP4"):
+        super().__init__()
+        self.ffn = w1.out_features
+        w13 = nn.Linear(w1.in_features, 2 * self.ffn, bias=False, device=w1.weight.device, dtype=torch.bfloat16)
+        w13.weight.data.copy_(torch.cat([w1.weight.data, w3.weight.data], dim=0))
+        self.w13 = QLinearLayer(w13, select_num, in_index, quant_type=quant_type)   # w1 and w3 share their input
+        self.w2 = QLinearLayer(w2, select_num, w2_index, quant_type=quant_type)
+        self.register_buffer("w1_reorder_index", in_index.to(torch.int16))
+        self.register_buffer("w2_reorder_index", w2_index.to(torch.int16))
+        self.quant_type = quant_type
+
+    @torch.no_grad()
+    def forward(self, x):
+        h = self.w13(quantize_tokens(x, self.w1_reorder_index, self.w13.select_num, self.quant_type))
+        t = F.silu(h[:, :self.ffn]) * h[:, self.ffn:]
+        return self.w2(quantize_tokens(t, self.w2_reorder_index, self.w2.select_num, self.quant_type))
+
+
+class MixtralSparseMoeBlock(nn.Module):
+    """model/qMixtralLayer.py:388-464: softmax router in fp32, top-k, renormalised weights, every
+    token processed by its experts without capacity limits."""
+
+    def __init__(self, gate: nn.Linear, experts, top_k=2):
+        super().__init__()
+        self.gate = gate
+        self.experts = nn.ModuleList(experts)
+        self.num_experts = len(experts)
+        self.top_k = top_k
+
+    @torch.no_grad()
+    def forward(self, hidden_states, router_logits: Optional[torch.Tensor] = None):
+        bsz, q_len, hid = hidden_states.shape
+        x = hidden_states.reshape(-1, hid)
+        if router_logits is None:
+            router_logits = self.gate(x)
+        w = F.softmax(router_logits, dim=1, dtype=torch.float)
+        w, sel = torch.topk(w, self.top_k, dim=-1)
+        w = (w / w.sum(dim=-1, keepdim=True)).to(x.dtype)
+        # (token, slot) pairs sorted by expert: one contiguous run of rows per expert
+        flat_e = sel.reshape(-1)
+        order = torch.argsort(flat_e, stable=True)
+        tok = order // self.top_k
+        counts = torch.bincount(flat_e, minlength=self.num_experts).tolist()   # the one host read-back
+        xs = x.index_select(0, tok)
+        ws = w.reshape(-1).index_select(0, order)
+        out = torch.zeros_like(x)
+        beg = 0
+        for e, n in enumerate(counts):
+            if n == 0:
+                continue
+            y = self.experts[e](xs[beg:beg + n].contiguous()) * ws[beg:beg + n, None]
+            out.index_add_(0, tok[beg:beg + n], y.to(x.dtype))
+            beg += n
+        return out.reshape(bsz, q_len, hid), router_logits
+
+
+def build_mixtral_block(hidden=4096, ffn=14336, num_experts=8, top_k=2, select_num=128, quant_type="NVFP4",
+                        indices=None, seed=5, device="cuda"):
+    """Random-weight MoE block of benchmark configuration 5; `indices[e]` = (input index, w2 index)."""
+    gen = torch.Generator().manual_seed(seed)
+    gate = _linear(num_experts, hidden, 1.0 / math.sqrt(hidden), device, gen)
+    experts = []
+    for e in range(num_experts):
+        w1 = _linear(ffn, hidden, 0.02, device, gen)
+        w3 = _linear(ffn, hidden, 0.02, device, gen)
+        w2 = _linear(hidden, ffn, 0.02, device, gen)
+        if indices is not None:
+            i_in, i_w2 = indices[e]
+        else:
+            i_in = torch.arange(hidden, dtype=torch.int16, device=device)
+            i_w2 = torch.arange(ffn, dtype=torch.int16, device=device)
+        experts.append(MixtralExpertMLP(w1, w3, w2, select_num, i_in, i_w2, quant_type))
+        del w1, w3, w2
+    return MixtralSparseMoeBlock(gate, experts, top_k)
