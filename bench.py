@@ -155,6 +155,119 @@ def gemm_rows(torch, agemm, shapes, Ms, fmts, iters=40):
     return rows
 
 
+def layer_rows(torch, iters=10):
+    """Benchmark configurations 4 and 5 through arcquant_amd.layers, next to the same layer in bf16
+    (torch: hipBLASLt GEMMs, the same SDPA).  One decoder layer of Llama-3-8B geometry (hidden 4096,
+    32 query / 8 KV heads of 128, SwiGLU 14336, fused qkv and gate_up), prefill 8 x 2048 tokens and a
+    decode step of batch 64 over a 2048-token KV cache; one Mixtral MoE block (8 experts, top-2,
+    4096 tokens, expert popularity Zipf(1.1))."""
+    import torch.nn.functional as F
+    from arcquant_amd import layers
+    rows = []
+    hidden, inter, nh, nkv, eps = 4096, 14336, 32, 8, 1e-5
+    d = hidden // nh
+    g = torch.Generator().manual_seed(4)
+
+    def hidden_states(b, s):
+        x = torch.randn(b, s, hidden, generator=g)
+        ch = torch.randperm(hidden, generator=g)[:41]
+        x[..., ch] *= 40.0
+        return x.to(torch.bfloat16).cuda()
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        return loop_time_ms(lambda i: fn(), iters, torch)
+
+    def rms(x, w):
+        h = x.float()
+        h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + eps)
+        return w * h.to(x.dtype)
+
+    for fmt in ("MXFP4", "NVFP4"):
+        layer = layers.LlamaDecoderLayer(hidden, inter, nh, nkv, eps=eps, select_num=256, select_num_down=256,
+                                         quant_type=fmt, seed=4)
+        W = {k: v.weight.data for k, v in layer.linears.items()}
+        g1, g2 = layer.input_layernorm.weight, layer.post_attention_layernorm.weight
+
+        def bf16_layer(x, kv=None, past=0):
+            b, s, _ = x.shape
+            qkv = F.linear(rms(x, g1), W["qkv"])
+            q = qkv[..., :nh * d].view(b, s, nh, d).transpose(1, 2)
+            k = qkv[..., nh * d:(nh + nkv) * d].view(b, s, nkv, d).transpose(1, 2)
+            v = qkv[..., (nh + nkv) * d:].view(b, s, nkv, d).transpose(1, 2)
+            q, k = layers.rotary_pos_emb(q, k, past)
+            if kv is not None:
+                kv[0][:, :, past:past + s] = k
+                kv[1][:, :, past:past + s] = v
+                k, v = kv[0][:, :, :past + s], kv[1][:, :, :past + s]
+            o = F.scaled_dot_product_attention(q, k, v, is_causal=(s > 1 and past == 0), enable_gqa=True)
+            h = x + F.linear(o.transpose(1, 2).reshape(b, s, hidden), W["o"])
+            gu = F.linear(rms(h, g2), W["gate_up"])
+            return h + F.linear(F.silu(gu[..., :inter]) * gu[..., inter:], W["down"])
+
+        x = hidden_states(8, 2048)
+        ms_arc = timed(lambda: layer(x))
+        ms_bf = timed(lambda: bf16_layer(x))
+        rows.append({"config": "decoder layer prefill 8x2048", "fmt": fmt, "arc_ms": round(ms_arc, 3),
+                     "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_arc, 2),
+                     "tokens_per_s": round(8 * 2048 / ms_arc * 1e3)})
+        print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
+        del x
+        kvlen = 2048
+        kv = (torch.randn(64, nkv, kvlen + 8, d, device="cuda", dtype=torch.bfloat16),
+              torch.randn(64, nkv, kvlen + 8, d, device="cuda", dtype=torch.bfloat16))
+        x = hidden_states(64, 1)
+        ms_arc = timed(lambda: layer(x, kv, kvlen))
+        ms_bf = timed(lambda: bf16_layer(x, kv, kvlen))
+        rows.append({"config": f"decoder layer decode batch 64, KV length {kvlen}", "fmt": fmt,
+                     "arc_ms": round(ms_arc, 3), "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_arc, 2),
+                     "tokens_per_s": round(64 / ms_arc * 1e3)})
+        print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
+        del layer, W, kv, x
+        torch.cuda.empty_cache()
+
+    # Mixtral block, NVFP4 (benchmark configuration 5), select_num 128
+    E, ffn, tokens = 8, 14336, 4096
+    g = torch.Generator().manual_seed(5)
+    block = layers.build_mixtral_block(hidden, ffn, E, 2, 128, "NVFP4", seed=5)
+    x = torch.randn(1, tokens, hidden, generator=g).to(torch.bfloat16).cuda()
+    bias = torch.log(1.0 / torch.arange(1, E + 1).float() ** 1.1)
+    logits = (torch.randn(tokens, E, generator=g) + bias).cuda()
+    ms_arc = timed(lambda: block(x, router_logits=logits))
+    # the same block in bf16 on dequantised-size weights (random: only the time matters)
+    w13 = [torch.randn(2 * ffn, hidden, device="cuda", dtype=torch.bfloat16) * 0.02 for _ in range(E)]
+    w2 = [torch.randn(hidden, ffn, device="cuda", dtype=torch.bfloat16) * 0.02 for _ in range(E)]
+
+    def bf16_moe():
+        xf = x.view(tokens, hidden)
+        w = F.softmax(logits, dim=1, dtype=torch.float)
+        w, sel = torch.topk(w, 2, dim=-1)
+        w = (w / w.sum(dim=-1, keepdim=True)).to(xf.dtype)
+        flat = sel.reshape(-1)
+        order = torch.argsort(flat, stable=True)
+        tok = order // 2
+        counts = torch.bincount(flat, minlength=E).tolist()
+        xs, ws = xf.index_select(0, tok), w.reshape(-1).index_select(0, order)
+        out = torch.zeros_like(xf)
+        beg = 0
+        for e, n in enumerate(counts):
+            if n:
+                h = F.linear(xs[beg:beg + n], w13[e])
+                y = F.linear(F.silu(h[:, :ffn]) * h[:, ffn:], w2[e]) * ws[beg:beg + n, None]
+                out.index_add_(0, tok[beg:beg + n], y)
+                beg += n
+        return out
+
+    ms_bf = timed(bf16_moe)
+    counts = torch.bincount(torch.topk(F.softmax(logits, dim=1), 2, dim=-1)[1].reshape(-1), minlength=E).tolist()
+    rows.append({"config": "Mixtral MoE block, 4096 tokens, 8 experts top-2", "fmt": "NVFP4", "arc_ms": round(ms_arc, 3),
+                 "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_arc, 2), "tokens_per_expert": counts,
+                 "tokens_per_s": round(tokens / ms_arc * 1e3)})
+    print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -162,6 +275,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--gemm-table", action="store_true", help="every benchmark GEMM shape x M (slower)")
     ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--layers", action="store_true", help="also time a decoder layer and an MoE block (configs 4, 5)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=M_TOKENS)
     args = ap.parse_args()
@@ -286,6 +400,8 @@ def main():
         Ms = [1, 16, 64, 128, 512, 2048, 4096] if args.gemm_table else [1, 16, 512, 4096]
         out["gemm"] = gemm_rows(torch, agemm, shapes, Ms, ["MXFP4", "NVFP4"])
         out["gemm_peaks_tflops"] = MFMA_PEAK_TFLOPS
+    if args.layers:
+        out["layers"] = layer_rows(torch)
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, args.cpu_rows)
