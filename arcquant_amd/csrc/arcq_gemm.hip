@@ -239,7 +239,8 @@ __device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (
   const int r = lane & 31, kh = lane >> 5;
   const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;
   const float alpha = effective_alpha(p);
-  if (m_base + BM <= p.M && n_base + BN <= p.N && (p.N & 7) == 0) {
+  constexpr bool kPow2 = (WN & (WN - 1)) == 0;  // the swizzled transpose below needs 4*WN lanes per row to be a power of two
+  if (kPow2 && m_base + BM <= p.M && n_base + BN <= p.N && (p.N & 7) == 0) {
     // Whole tile inside C: transpose each wave's tile through LDS (free now) so that every store
     // instruction writes whole rows of the wave tile, 16 bytes per lane.
     wait_dma_and_sync();  // every wave is done reading operands
@@ -457,10 +458,8 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
 // v_mfma_f32_32x32x16_f16.  Since the scale is applied per element, an MFMA K step need not be a
 // block: a lane reads one 16-byte chunk and feeds its four dwords (8 codes each) to four MFMAs,
 // lanes 0-31 from chunk 4*0+cp, lanes 32-63 from chunk 4*1+cp.
-// Decode of 8 codes (one dword): the 3-bit magnitudes index an 8-entry byte table of fp16 HIGH
-// bytes {00,38,3C,3E,40,42,44,46} (the low byte of those fp16 values is zero) through v_perm_b32,
-// the sign bits are or-ed in, bytes are spread to 16-bit lanes, and one packed fp16 multiply
-// applies the block scale: 16 VALU instructions per 8 values.
+// Decode of 8 codes (one dword): four v_cvt_scalef32_pk_f16_fp4 (two codes each, exact) and four
+// packed fp16 multiplies by the block scale: 8 VALU instructions per 8 values.
 // Requires K' % 128 == 0.
 // ---------------------------------------------------------------------------------------------
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -483,18 +482,13 @@ __device__ __forceinline__ uint32_t pk_mul_f16_bcast(uint32_t a, uint32_t s) {
 
 template <bool HI>
 __device__ __forceinline__ v8h decode8_nvfp4_f16(uint32_t codes, uint32_t scale_pair) {
-  const uint32_t lut_lo = 0x3e3c3800u, lut_hi = 0x46444240u;  // fp16 high bytes of 0,.5,1,1.5 | 2,3,4,6
-  const uint32_t se = codes & 0x07070707u;                    // magnitudes of elements 0,2,4,6
-  const uint32_t so = (codes >> 4) & 0x07070707u;             // 1,3,5,7
-  uint32_t he = __builtin_amdgcn_perm(lut_hi, lut_lo, se);
-  uint32_t ho = __builtin_amdgcn_perm(lut_hi, lut_lo, so);
-  he |= (codes << 4) & 0x80808080u;                           // signs (bit 3 of a nibble -> bit 7 of the byte)
-  ho |= codes & 0x80808080u;
+  // hardware FP4 -> fp16 conversion, two codes per instruction (low nibble first), then one packed
+  // multiply by the block scale: 8 VALU instructions per 8 values
   v4u d;
-  d[0] = __builtin_amdgcn_perm(ho, he, 0x040c000cu);          // {0, he.b0, 0, ho.b0}: elements 0,1 as fp16
-  d[1] = __builtin_amdgcn_perm(ho, he, 0x050c010cu);
-  d[2] = __builtin_amdgcn_perm(ho, he, 0x060c020cu);
-  d[3] = __builtin_amdgcn_perm(ho, he, 0x070c030cu);
+  d[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 0));
+  d[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 1));
+  d[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 2));
+  d[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 1.0f, 3));
 #pragma unroll
   for (int k = 0; k < 4; ++k) d[k] = pk_mul_f16_bcast<HI>(d[k], scale_pair);
   return __builtin_bit_cast(v8h, d);
@@ -656,7 +650,7 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
 #pragma unroll
       for (int g = 0; g < WN * WM; ++g) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, (16 * (WN + WM) + WN * WM - 1) / (WN * WM), 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, (8 * (WN + WM) + WN * WM - 1) / (WN * WM), 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -935,6 +929,7 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
   if (fmt == ARCQ_FMT_NVFP4 && force != 0 && fast_ok) {
     if (force == 44 || (force < 0 && M > 1024)) return launch_nvfp4_tiled<4, 4>(p, st);
     if (force == 42) return launch_nvfp4_tiled<4, 2>(p, st);
+    if (force == 34) return launch_nvfp4_tiled<3, 4>(p, st);
     if (force == 22 || (force < 0 && M > 128)) return launch_nvfp4_tiled<2, 2>(p, st);
     if (force == 21 || force < 0) return launch_nvfp4_tiled<2, 1>(p, st);
   }
