@@ -30,7 +30,8 @@ import torch
 from . import _lib
 from ._lib import FORMATS, ArcqError  # noqa: F401
 
-__all__ = ["matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "dequantize", "check_index",
+__all__ = ["matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "swiglu_quantize_x", "dequantize",
+           "check_index",
            "unpack_codes", "scale_values"]
 
 
@@ -121,6 +122,49 @@ def reorder_quantize_w(W, reorder_index, KE, *, fmt="NVFP4", global_scale=None):
 def rmsnorm_quantize_x(X, W, eps, reorder_index, KE, *, fmt="NVFP4", global_scale=None):
     """agemm.rmsnorm_quantize_x (kernels/src/bindings.cpp:216-254); W is the RMSNorm weight bf16 [K]."""
     return _quantize("arcq_rmsnorm_quantize_x", X, W, eps, reorder_index, KE, fmt, global_scale)
+
+
+def swiglu_quantize_x(gate, up, reorder_index, KE, *, fmt="NVFP4", global_scale=None):
+    """act_fn(gate) * up -> quantized activations in one pass (no counterpart in the reference's
+    module; its layers do silu, multiply and quantize as separate ops, model/qLlamaLayer.py:432-439).
+    gate, up: bf16 [M, K] views with the same row stride and unit column stride, e.g. the two
+    halves of a fused gate_up output.  global_scale: None / float / 0-dim CUDA tensor;
+    "absmax" computes the NVFP4 tensor scale max|t| / 2688 on the device first and returns it
+    as a third value."""
+    f = _fmt_id(fmt)
+    L = _lib.lib()
+    for t, name in ((gate, "gate"), (up, "up")):
+        if not isinstance(t, torch.Tensor) or t.dtype != torch.bfloat16 or not t.is_cuda or t.dim() != 2:
+            raise RuntimeError(f"{name} must be a 2-D bf16 CUDA tensor")
+        if t.stride(1) != 1:
+            raise RuntimeError(f"{name} must have unit stride along its last dimension")
+    if gate.shape != up.shape or gate.stride(0) != up.stride(0) or gate.device != up.device:
+        raise RuntimeError("gate and up must have the same shape, row stride and device")
+    _require(reorder_index, "reorder_index", torch.int16, 1)
+    M, K = gate.shape
+    ld = gate.stride(0) if M > 1 else K
+    KE = int(KE)
+    G = L.arcq_group_size(f)
+    if K % 32 or K < 32 or K > 16384 or KE < 0 or KE > K or KE % G or reorder_index.numel() != K or ld % 8:
+        raise RuntimeError(f"Value error in swiglu_quantize_x: K={K}, KE={KE}, row stride {ld} not supported for {fmt}")
+    want_scale = isinstance(global_scale, str)
+    with torch.cuda.device(gate.device):
+        if want_scale:
+            if global_scale != "absmax":
+                raise RuntimeError("global_scale must be a number, a tensor or 'absmax'")
+            amax = torch.zeros((), dtype=torch.float32, device=gate.device)
+            _lib.check(L.arcq_swiglu_absmax(gate.data_ptr(), up.data_ptr(), ld, M, K, amax.data_ptr(), _stream(gate)),
+                       "arcq_swiglu_absmax")
+            global_scale = amax / torch.full_like(amax, 2688.0)
+            global_scale = torch.where(global_scale == 0, torch.ones_like(global_scale), global_scale)
+        gs, d_gs, keep = _scalar(global_scale, gate.device)
+        QX = torch.empty((M, (K + KE) // 2), dtype=torch.uint8, device=gate.device)
+        SFX = torch.empty((L.arcq_scales_bytes(M, K, KE, f),), dtype=torch.uint8, device=gate.device)
+        rc = L.arcq_swiglu_quantize_x(gate.data_ptr(), up.data_ptr(), ld, M, K, reorder_index.data_ptr(), KE, f, gs,
+                                      d_gs, QX.data_ptr(), SFX.data_ptr(), _stream(gate))
+    _lib.check(rc, "arcq_swiglu_quantize_x")
+    del keep
+    return (QX, SFX, global_scale) if want_scale else (QX, SFX)
 
 
 def _infer_fmt(A, SFA, fmt):

@@ -15,7 +15,7 @@
 namespace arcq {
 namespace {
 
-enum { MODE_X = 0, MODE_W = 1, MODE_NORM = 2 };
+enum { MODE_X = 0, MODE_W = 1, MODE_NORM = 2, MODE_SWIGLU = 3 };
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains outstanding
 // global loads and stores (s_waitcnt vmcnt(0)), which would serialise the next row's prefetch
@@ -30,6 +30,8 @@ constexpr int kThreads = 256;
 struct QuantParams {
   const uint16_t *x;      // bf16 [rows, K]
   const uint16_t *gamma;  // bf16 [K] (MODE_NORM)
+  const uint16_t *up;     // bf16 rows of the "up" operand (MODE_SWIGLU; x holds the "gate" rows)
+  int ldx;                // row stride of x (and up) in elements; K except for MODE_SWIGLU
   const int16_t *idx;     // [K]
   uint8_t *codes;         // [rows, (K+S)/2]
   uint8_t *scales;        // [rows, (K+S)/G]
@@ -242,9 +244,9 @@ __device__ __forceinline__ float scale_rcp(float s) {
 // gamma * h for the two bf16 halves of one register: v_dot2_f32_bf16 with the other half of the
 // gamma operand zeroed gives the exact fp32 product without unpacking h
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b) {
-  float d;
-  asm("v_dot2_f32_bf16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
-  return d;
+  // the builtin, not inline asm: the compiler then sees the instruction and keeps the wait states
+  // it needs after the VALU instructions that produce its operands
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, a), __builtin_bit_cast(v2bf, b), 0.0f, false);
 }
 
 // Sum of one double per lane over the 64 lanes of a wave, in DPP register moves (no LDS round
@@ -340,6 +342,15 @@ __device__ __forceinline__ void unit_exact(const uint32_t (&yv)[16], float g, ui
   }
 }
 
+// act_fn(gate) * up as the reference's layers form it in bf16 (model/qLlamaLayer.py:432,
+// model/qMixtralLayer.py:531): SiLU evaluated in fp32 as x / (1 + exp(-x)) and rounded to bf16,
+// then a bf16 multiply (fp32 product, one rounding).  Two elements per call, packed.
+__device__ __forceinline__ uint32_t swiglu_pair(uint32_t gw, uint32_t uw) {
+  const float g0 = u2f(gw << 16), g1 = u2f(gw & 0xffff0000u);
+  const uint32_t a = pack_bf16_rne(g0 / (1.0f + expf(-g0)), g1 / (1.0f + expf(-g1)));
+  return pack_bf16_rne(dot2_bf16(a, uw & 0xffffu), dot2_bf16(a, uw & 0xffff0000u));
+}
+
 template <int FMT, int MODE, bool SCALED>
 __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p) {
   extern __shared__ uint4 smem[];
@@ -371,11 +382,17 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
   const bool eps_normal = p.eps >= 0x1p-90f;
 
   int r = blockIdx.x;
-  uint4 q0 = make_uint4(0, 0, 0, 0), q1 = q0;
+  const size_t ldx = MODE == MODE_SWIGLU ? (size_t)p.ldx : (size_t)K;
+  uint4 q0 = make_uint4(0, 0, 0, 0), q1 = q0, u0 = q0, u1 = q0;
   if (r < p.rows && active) {  // first row in flight before anything that has to wait for memory
-    const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)r * K);
+    const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)r * ldx);
     q0 = src[tid];
     q1 = src[tid + nunits];
+    if (MODE == MODE_SWIGLU) {
+      const uint4 *usrc = reinterpret_cast<const uint4 *>(p.up + (size_t)r * ldx);
+      u0 = usrc[tid];
+      u1 = usrc[tid + nunits];
+    }
   }
 
   // channel-only state, loaded once
@@ -410,11 +427,16 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
   for (int i = 0; i < 16; ++i) yv[i] = 0u;  // low halves stay zero: only d16_hi loads write these
 
   for (; r < p.rows; r += gridDim.x) {
-    uint4 n0 = q0, n1 = q1;
+    uint4 n0 = q0, n1 = q1, un0 = u0, un1 = u1;
     if (r + (int)gridDim.x < p.rows && active) {  // prefetch the next row of this workgroup
-      const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)(r + gridDim.x) * K);
+      const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)(r + gridDim.x) * ldx);
       n0 = src[tid];
       n1 = src[tid + nunits];
+      if (MODE == MODE_SWIGLU) {
+        const uint4 *usrc = reinterpret_cast<const uint4 *>(p.up + (size_t)(r + gridDim.x) * ldx);
+        un0 = usrc[tid];
+        un1 = usrc[tid + nunits];
+      }
     }
     if (MODE == MODE_NORM) {
       const uint32_t xw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
@@ -464,6 +486,16 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
       if (active) {
         reinterpret_cast<uint4 *>(row)[tid] = make_uint4(yw[0], yw[1], yw[2], yw[3]);
         reinterpret_cast<uint4 *>(row)[tid + nunits] = make_uint4(yw[4], yw[5], yw[6], yw[7]);
+      }
+    } else if (MODE == MODE_SWIGLU) {
+      const uint4 t0 = make_uint4(swiglu_pair(q0.x, u0.x), swiglu_pair(q0.y, u0.y), swiglu_pair(q0.z, u0.z),
+                                  swiglu_pair(q0.w, u0.w));
+      const uint4 t1 = make_uint4(swiglu_pair(q1.x, u1.x), swiglu_pair(q1.y, u1.y), swiglu_pair(q1.z, u1.z),
+                                  swiglu_pair(q1.w, u1.w));
+      lds_barrier();  // the previous row's gathers are over
+      if (active) {
+        reinterpret_cast<uint4 *>(row)[tid] = t0;
+        reinterpret_cast<uint4 *>(row)[tid + nunits] = t1;
       }
     } else {
       lds_barrier();  // the previous row's gathers are over
@@ -538,7 +570,38 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
     }
     q0 = n0;
     q1 = n1;
+    if (MODE == MODE_SWIGLU) {
+      u0 = un0;
+      u1 = un1;
+    }
   }
+}
+
+// max |act_fn(gate) * up| over the whole tensor (the NVFP4 tensor scale's numerator,
+// model/qLlamaLayer.py:74), as the fp32 bits of a non-negative value: atomicMax on them is a max
+__global__ __launch_bounds__(256) void swiglu_absmax_kernel(const uint16_t *gate, const uint16_t *up, size_t ld, int rows,
+                                                            int K, uint32_t *out) {
+  const int cpr = K >> 3;  // 16-byte chunks per row
+  const size_t total = (size_t)rows * cpr;
+  uint32_t m = 0u;
+  for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < total; c += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = c / cpr, k = (c % cpr) << 3;
+    const uint4 g = *reinterpret_cast<const uint4 *>(gate + r * ld + k);
+    const uint4 u = *reinterpret_cast<const uint4 *>(up + r * ld + k);
+    const uint32_t t[4] = {swiglu_pair(g.x, u.x), swiglu_pair(g.y, u.y), swiglu_pair(g.z, u.z), swiglu_pair(g.w, u.w)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t lo = (t[i] << 16) & 0x7fffffffu, hi = t[i] & 0x7fff0000u;
+      m = lo > m ? lo : m;
+      m = hi > m ? hi : m;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint32_t v = (uint32_t)__shfl_xor((int)m, o);
+    m = v > m ? v : m;
+  }
+  if ((threadIdx.x & 63) == 0 && m) atomicMax(out, m);
 }
 
 template <int FMT, int MODE, bool SCALED>
@@ -643,6 +706,8 @@ int quantize_entry(int mode, const void *x, const void *gamma, float eps, int ro
   p.K = K;
   p.S = S;
   p.inv_k = 1.0 / (double)K;
+  p.up = nullptr;
+  p.ldx = K;
   hipStream_t st = static_cast<hipStream_t>(stream);
   // tensor scale known on the host to be 1: operands are exactly bf16 -> fast kernels
   if (!d_gscale && gscale == 1.0f && K <= 16384) {
@@ -672,6 +737,39 @@ int quantize_entry(int mode, const void *x, const void *gamma, float eps, int ro
   if (mode == MODE_X) return launch_quantize<ARCQ_FMT_MXFP4, MODE_X>(p, st);
   if (mode == MODE_W) return launch_quantize<ARCQ_FMT_MXFP4, MODE_W>(p, st);
   return launch_quantize<ARCQ_FMT_MXFP4, MODE_NORM>(p, st);
+}
+
+int swiglu_entry(const void *gate, const void *up, int ld, int rows, int K, const int16_t *idx, int S, int fmt,
+                 float gscale, const float *d_gscale, void *codes, void *scales, void *stream) {
+  if (fmt != ARCQ_FMT_NVFP4 && fmt != ARCQ_FMT_MXFP4) return ARCQ_ERR_FORMAT;
+  const int G = arcq_group_size(fmt);
+  if (rows < 0 || K < 32 || K % 32 != 0 || K > 16384 || S < 0 || S > K || S % G != 0 || ld < K || ld % 8 != 0)
+    return ARCQ_ERR_SHAPE;
+  if (rows == 0) return ARCQ_OK;
+  if (!gate || !up || !idx || !codes || !scales) return ARCQ_ERR_NULL;
+  if (!aligned16(gate) || !aligned16(up) || !aligned16(idx) || !aligned16(codes)) return ARCQ_ERR_ALIGN;
+  QuantParams p;
+  p.x = static_cast<const uint16_t *>(gate);
+  p.up = static_cast<const uint16_t *>(up);
+  p.ldx = ld;
+  p.gamma = nullptr;
+  p.idx = idx;
+  p.codes = static_cast<uint8_t *>(codes);
+  p.scales = static_cast<uint8_t *>(scales);
+  p.d_gscale = d_gscale;
+  p.gscale = gscale;
+  p.eps = 0.0f;
+  p.rows = rows;
+  p.K = K;
+  p.S = S;
+  p.inv_k = 0.0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool unit = !d_gscale && gscale == 1.0f;
+  if (fmt == ARCQ_FMT_NVFP4)
+    return unit ? launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_SWIGLU, false>(p, st)
+                : launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_SWIGLU, true>(p, st);
+  return unit ? launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_SWIGLU, false>(p, st)
+              : launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_SWIGLU, true>(p, st);
 }
 
 }  // namespace
@@ -727,6 +825,27 @@ int arcq_check_index(const int16_t *reorder_index, int K, void *stream) {
   (void)hipFree(d_bad);
   if (e != hipSuccess) return arcq::note_hip_error(e);
   return bad ? ARCQ_ERR_INDEX : ARCQ_OK;
+}
+
+int arcq_swiglu_quantize_x(const void *gate, const void *up, int ld, int M, int K, const int16_t *reorder_index,
+                           int select_num, int fmt, float global_scale, const float *d_global_scale, void *codes,
+                           void *scales, void *stream) {
+  return arcq::swiglu_entry(gate, up, ld, M, K, reorder_index, select_num, fmt, global_scale, d_global_scale, codes,
+                            scales, stream);
+}
+
+int arcq_swiglu_absmax(const void *gate, const void *up, int ld, int M, int K, float *d_absmax, void *stream) {
+  if (M < 0 || K < 8 || K % 8 != 0 || ld < K || ld % 8 != 0) return ARCQ_ERR_SHAPE;
+  if (M == 0) return ARCQ_OK;
+  if (!gate || !up || !d_absmax) return ARCQ_ERR_NULL;
+  if (!arcq::aligned16(gate) || !arcq::aligned16(up)) return ARCQ_ERR_ALIGN;
+  const size_t chunks = (size_t)M * (K >> 3);
+  const int grid = (int)((chunks + 255) / 256 < 4096 ? (chunks + 255) / 256 : 4096);
+  hipLaunchKernelGGL(arcq::swiglu_absmax_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t *>(gate), static_cast<const uint16_t *>(up), (size_t)ld, M, K,
+                     reinterpret_cast<uint32_t *>(d_absmax));
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
 }
 
 int arcq_stream_probe(const void *src, void *dst, size_t bytes_in, size_t bytes_out, void *stream) {

@@ -59,6 +59,26 @@ def reorder_quantize_x(x, reorder_index, select_num, quant_type="NVFP4"):
     return qx, scale_x, 1.0
 
 
+def swiglu_quantize_tokens(gate_up, inter, reorder_index, select_num, quant_type="NVFP4"):
+    """act_fn(gate) * up -> quantized tuple in one fused pass over the output of a fused gate_up
+    projection ([..., 2*inter]: gate first).  Same values as quantize_tokens(F.silu(gate) * up, ...),
+    without the [tokens, inter] intermediate going through memory three times."""
+    if gate_up.dim() == 3:
+        bsz, q_len, _ = gate_up.shape
+        flat = gate_up.reshape(bsz * q_len, -1)
+    else:
+        bsz, q_len = None, gate_up.shape[0]
+        flat = gate_up
+    gate, up = flat[:, :inter], flat[:, inter:]
+    if quant_type == "NVFP4":
+        qx, sfx, scale = agemm.swiglu_quantize_x(gate, up, reorder_index, select_num, fmt="NVFP4",
+                                                 global_scale="absmax")
+    else:
+        qx, sfx = agemm.swiglu_quantize_x(gate, up, reorder_index, select_num, fmt=quant_type)
+        scale = 1.0
+    return qx, sfx, scale, bsz, q_len
+
+
 def quantize_tokens(hidden_states, reorder_index, select_num, quant_type="NVFP4"):
     """[bsz, q_len, K] or [tokens, K] -> the 5-tuple a QLinearLayer takes."""
     if hidden_states.dim() == 3:
@@ -174,6 +194,9 @@ class LlamaMLP(nn.Module):
     def forward(self, x):
         """x: the tuple of the already quantized (normalised) hidden states"""
         gu = self.gate_up_proj(x)
+        if self.inter <= 16384 and self.inter % 32 == 0:
+            return self.down_proj(swiglu_quantize_tokens(gu, self.inter, self.down_reorder_index,
+                                                         self.down_proj.select_num, self.quant_type))
         t = F.silu(gu[..., :self.inter]) * gu[..., self.inter:]
         return self.down_proj(quantize_tokens(t, self.down_reorder_index, self.down_proj.select_num, self.quant_type))
 
@@ -267,6 +290,9 @@ class MixtralExpertMLP(nn.Module):
     @torch.no_grad()
     def forward(self, x):
         h = self.w13(quantize_tokens(x, self.w1_reorder_index, self.w13.select_num, self.quant_type))
+        if self.ffn <= 16384 and self.ffn % 32 == 0:
+            return self.w2(swiglu_quantize_tokens(h, self.ffn, self.w2_reorder_index, self.w2.select_num,
+                                                  self.quant_type))
         t = F.silu(h[:, :self.ffn]) * h[:, self.ffn:]
         return self.w2(quantize_tokens(t, self.w2_reorder_index, self.w2.select_num, self.quant_type))
 

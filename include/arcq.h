@@ -103,6 +103,23 @@ int arcq_rmsnorm_quantize_x(const void *x, const void *gamma, float eps, int M, 
                             const float *d_global_scale, void *codes, void *scales, void *stream);
 
 /*
+ * Fused SwiGLU + activation quantizer for the down projection's input: t = act_fn(gate) * up
+ * formed as the reference's layers form it in bf16 -- SiLU in fp32 as g / (1 + exp(-g)), rounded to
+ * bf16, times up, rounded to bf16 (model/qLlamaLayer.py:432, model/qMixtralLayer.py:531) -- and
+ * quantized like arcq_reorder_quantize_x without t ever reaching memory.  The reference names this
+ * fusion but does not ship it (benchmarks/modeling_arc.py:112, commented activate_quantize_x).
+ *   gate, up  bf16 rows of K elements with a common row stride `ld` (elements, multiple of 8): for a
+ *             fused gate_up projection output [M, 2K] pass up = gate + K and ld = 2K
+ *   K         multiple of 32, 32 <= K <= 16384
+ * arcq_swiglu_absmax computes max |t| over the tensor (numerator of the NVFP4 tensor scale,
+ * model/qLlamaLayer.py:74) into *d_absmax, which the caller has set to 0; nothing synchronises.
+ */
+int arcq_swiglu_quantize_x(const void *gate, const void *up, int ld, int M, int K, const int16_t *reorder_index,
+                           int select_num, int fmt, float global_scale, const float *d_global_scale, void *codes,
+                           void *scales, void *stream);
+int arcq_swiglu_absmax(const void *gate, const void *up, int ld, int M, int K, float *d_absmax, void *stream);
+
+/*
  * Augmented-K block-scaled FP4 GEMM: C[M,N] = alpha * dq(A)[M,K'] @ dq(B)[N,K']^T, fp32
  * accumulation, bf16 output.
  * Replaces agemm.matmul (kernels/src/bindings.cpp:99-120 -> nvfp4.cu:35-132).
