@@ -35,8 +35,8 @@ H, M_TOKENS, SELECT, EPS = 4096, 4096, 256, 1e-5
 FMT = "NVFP4"
 # HBM bytes per launch of the headline kernel on this workload from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (two runs), each scaled by what the same counter reads for arcq_stream_probe moving a known
-# number of bytes (profiles/bench_quantize_and_gemm_kernels.md): 33.76 MB fetched + 10.09 MB written.
-MEASURED_TRAFFIC_BYTES = 43_850_000
+# number of bytes (profiles/bench_quantize_and_gemm_kernels.md): 33.74 MB fetched + 10.09 MB written.
+MEASURED_TRAFFIC_BYTES = 43_830_000
 
 
 def quant_bytes(M, K, S, fmt, fused_norm):
