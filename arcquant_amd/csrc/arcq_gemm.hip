@@ -920,10 +920,18 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
     return fmt == ARCQ_FMT_MXFP4 ? launch_skinny_for<ARCQ_FMT_MXFP4>(p, st) : launch_skinny_for<ARCQ_FMT_NVFP4>(p, st);
   }
   if (fmt == ARCQ_FMT_MXFP4 && force != 0 && fast_ok) {
-    if (force == 44) return launch_mxfp4_tiled<4, 4>(p, st);
-    if (force == 42 || (force < 0 && M > 1024)) return launch_mxfp4_tiled<4, 2>(p, st);
+    // Tile choice from a small cost model: rounds of resident workgroups x cost of one round.
+    // 256x256 tiles run ~1.3x faster per flop than 256x128 ones (LDS reads per MFMA) and 128x128
+    // ones ~0.75x; 128x128 workgroups fit two to a CU.  Units: a 256x128 tile = 2.
+    const long t44 = (long)((M + 255) / 256) * ((N + 255) / 256), t42 = (long)((M + 127) / 128) * ((N + 255) / 256);
+    const long t22 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    const double c44 = (double)((t44 + 255) / 256) * 3.08, c42 = (double)((t42 + 255) / 256) * 2.0;
+    const double c22 = t22 <= 256 ? 1.33 : (double)((t22 + 511) / 512) * 2.67;
+    const int pick = M <= 128 ? 21 : (M < 512 ? 22 : (c44 < c42 && c44 < c22 ? 44 : (c42 <= c22 ? 42 : 22)));
+    if (force == 44 || (force < 0 && pick == 44)) return launch_mxfp4_tiled<4, 4>(p, st);
+    if (force == 42 || (force < 0 && pick == 42)) return launch_mxfp4_tiled<4, 2>(p, st);
     if (force == 24) return launch_mxfp4_tiled<2, 4>(p, st);
-    if (force == 22 || (force < 0 && M > 128)) return launch_mxfp4_tiled<2, 2>(p, st);
+    if (force == 22 || (force < 0 && pick == 22)) return launch_mxfp4_tiled<2, 2>(p, st);
     if (force == 21 || force < 0) return launch_mxfp4_tiled<2, 1>(p, st);
   }
   if (fmt == ARCQ_FMT_NVFP4 && force != 0 && fast_ok) {
