@@ -53,12 +53,16 @@ def lib() -> ctypes.CDLL:
     L.arcq_rmsnorm_quantize_x.argtypes = [vp, vp, f, i, i, vp, i, i, f, vp, vp, vp, vp]
     L.arcq_swiglu_quantize_x.argtypes = [vp, vp, i, i, i, vp, i, i, f, vp, vp, vp, vp]
     L.arcq_swiglu_absmax.argtypes = [vp, vp, i, i, i, vp, vp]
+    L.arcq_kv_append_i4.argtypes = [vp, vp, i, i, vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
+    L.arcq_kv_store_i4.argtypes = [vp, vp, vp, vp, i, vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
+    L.arcq_kv_decode_i4.argtypes = [vp, vp, i, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, f, vp]
     L.arcq_matmul.argtypes = [vp, vp, vp, vp, i, i, i, i, f, vp, vp, vp, vp]
     L.arcq_check_index.argtypes = [vp, i, vp]
     L.arcq_dequantize.argtypes = [vp, vp, i, i, i, vp, vp]
     L.arcq_stream_probe.argtypes = [vp, vp, sz, sz, vp]
     for name in ("arcq_reorder_quantize_x", "arcq_reorder_quantize_w", "arcq_rmsnorm_quantize_x", "arcq_matmul",
-                 "arcq_check_index", "arcq_dequantize", "arcq_stream_probe", "arcq_swiglu_quantize_x", "arcq_swiglu_absmax"):
+                 "arcq_check_index", "arcq_dequantize", "arcq_stream_probe", "arcq_swiglu_quantize_x", "arcq_swiglu_absmax",
+                 "arcq_kv_append_i4", "arcq_kv_store_i4", "arcq_kv_decode_i4"):
         getattr(L, name).restype = i
     _lib = L
     return L

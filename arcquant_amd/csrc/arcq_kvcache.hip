@@ -1,0 +1,388 @@
+// INT4 paged KV cache: quantize + append, and batched decode attention over the quantized pages.
+//
+// Replaces the reference's agemm.init_kv_i4 / append_kv_i4 / batch_decode_i4
+// (kernels/src/bindings.cpp:287-413 -> kernels/src/flashinfer.cu:9-112, a thin wrapper around a
+// patched FlashInfer that is not part of the reference tree) together with the torch-side quantizer
+// asym_quantize_and_pack_i4 (model/kv_cache.py:23-37), which is fused into the append here.
+//
+// Container layout = the reference's (model/kv_cache.py:148-160):
+//   kv_data   u8  [pages, n_layers, 2 (k, v), kv_heads, page_size, head_dim / 2]   element 2j in the low nibble
+//   kv_param  T2  [pages, n_layers, 2,        kv_heads, page_size, 2]              (scale, zero) in the model dtype T
+//   kv_indptr int32 [batch + 1], kv_indices int32 [kv_indptr[batch]], last_page_offset int32 [batch]:
+//   sequence b owns pages kv_indices[kv_indptr[b] .. kv_indptr[b+1]) in order and holds
+//   (pages_b - 1) * page_size + last_page_offset[b] tokens.
+// A stored value n (0..15) of a (token, head) row stands for n * scale - zero (kv_cache.py:39-43).
+//
+// head_dim is 128 (the only instantiation of the reference, flashinfer.cu:212-223).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/arcq.h"
+#include "arcq_internal.h"
+#include "arcq_math.h"
+
+namespace arcq {
+namespace {
+
+constexpr int kHeadDim = 128;
+constexpr int kRowBytes = kHeadDim / 2;  // one (token, head) row of codes
+
+struct KvLayout {
+  uint8_t *data;
+  uint32_t *param;  // two T values per row
+  const int32_t *indptr, *indices, *last_page_offset;
+  int n_layers, layer, heads, page_size;
+};
+
+// row index of (page, k_or_v, head, slot) in units of one (token, head) row
+__device__ __forceinline__ size_t kv_row(const KvLayout &c, int page, int kv, int head, int slot) {
+  return ((((size_t)page * c.n_layers + c.layer) * 2 + kv) * c.heads + head) * c.page_size + slot;
+}
+
+__device__ __forceinline__ float half_bits_to_f32(uint32_t h) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+__device__ __forceinline__ uint32_t f32_to_half_bits(float f) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);  // round to nearest even
+}
+template <bool BF16>
+__device__ __forceinline__ float rn(float f) {  // one torch elementwise op's result in the tensor dtype
+  return BF16 ? bf16_bits_to_f32(f32_to_bf16_bits(f)) : half_bits_to_f32(f32_to_half_bits(f));
+}
+template <bool BF16>
+__device__ __forceinline__ float from_bits(uint32_t b) {
+  return BF16 ? bf16_bits_to_f32(b & 0xffffu) : half_bits_to_f32(b & 0xffffu);
+}
+template <bool BF16>
+__device__ __forceinline__ uint32_t to_bits(float f) {
+  return BF16 ? f32_to_bf16_bits(f) : f32_to_half_bits(f);
+}
+
+// all-reduce over the 16 lanes of a DPP row
+#define ARCQ_ROW_XCHG(x, ctrl) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), ctrl, 0xf, 0xf, true))
+__device__ __forceinline__ float row16_sum(float v) {
+  v += ARCQ_ROW_XCHG(v, 0xb1);   // quad_perm [1,0,3,2]
+  v += ARCQ_ROW_XCHG(v, 0x4e);   // quad_perm [2,3,0,1]
+  v += ARCQ_ROW_XCHG(v, 0x141);  // row_half_mirror
+  v += ARCQ_ROW_XCHG(v, 0x140);  // row_mirror
+  return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, ARCQ_ROW_XCHG(v, 0xb1));
+  v = fmaxf(v, ARCQ_ROW_XCHG(v, 0x4e));
+  v = fmaxf(v, ARCQ_ROW_XCHG(v, 0x141));
+  v = fmaxf(v, ARCQ_ROW_XCHG(v, 0x140));
+  return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// append: quantize new (token, head) rows of K and V and scatter them into their pages.
+// asym_quantize_and_pack_i4 (model/kv_cache.py:23-37), every torch op rounded to the tensor dtype:
+//   scale = (max - min).clamp(min=1e-5) / 15 ; zero = -min ; q = clamp(round((x + zero) / scale), 0, 15)
+// 16 lanes per row (8 values each), one wave = 4 rows.
+// ---------------------------------------------------------------------------------------------
+template <bool BF16>
+__device__ __forceinline__ void quantize_row_store(const uint16_t *src, const KvLayout &c, size_t row, int lane16) {
+  const uint4 raw = reinterpret_cast<const uint4 *>(src)[lane16];
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  float x[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x[2 * i] = from_bits<BF16>(w[i]);
+    x[2 * i + 1] = from_bits<BF16>(w[i] >> 16);
+  }
+  float mx = x[0], mn = x[0];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) {
+    mx = fmaxf(mx, x[i]);
+    mn = fminf(mn, x[i]);
+  }
+  mx = row16_max(mx);
+  mn = -row16_max(-mn);
+  float d = rn<BF16>(mx - mn);
+  d = d < 1e-5f ? rn<BF16>(1e-5f) : d;
+  const float scale = rn<BF16>(d / 15.0f);
+  const float zero = -mn;
+  uint32_t packed = 0u;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float t = rn<BF16>(rn<BF16>(x[i] + zero) / scale);
+    const float r = fminf(fmaxf(rintf(t), 0.0f), 15.0f);  // torch.round: half to even
+    packed |= (uint32_t)r << (4 * i);
+  }
+  reinterpret_cast<uint32_t *>(c.data + row * kRowBytes)[lane16] = packed;
+  if (lane16 == 0) c.param[row] = to_bits<BF16>(scale) | (to_bits<BF16>(zero) << 16);
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void kv_append_i4_kernel(const uint16_t *k, const uint16_t *v, const int32_t *seq_indptr,
+                                                           KvLayout c) {
+  const int b = blockIdx.x;
+  const int tok0 = seq_indptr ? seq_indptr[b] : b;                 // first new token of this sequence in k / v
+  const int n_new = seq_indptr ? seq_indptr[b + 1] - tok0 : 1;
+  const int p0 = c.indptr[b], np = c.indptr[b + 1] - p0;
+  const int len = (np - 1) * c.page_size + c.last_page_offset[b];  // length after the append
+  const int lane16 = threadIdx.x & 15;
+  const int rows = n_new * c.heads;
+  for (int r = blockIdx.y * 16 + (threadIdx.x >> 4); r < rows; r += gridDim.y * 16) {
+    const int i = r / c.heads, head = r - i * c.heads;
+    const int pos = len - n_new + i;
+    const int page = c.indices[p0 + pos / c.page_size], slot = pos % c.page_size;
+    const size_t src = ((size_t)(tok0 + i) * c.heads + head) * kHeadDim;
+    quantize_row_store<BF16>(k + src, c, kv_row(c, page, 0, head, slot), lane16);
+    quantize_row_store<BF16>(v + src, c, kv_row(c, page, 1, head, slot), lane16);
+  }
+}
+
+// the same scatter for rows a caller has quantized already (what the reference's init_kv_i4 /
+// append_kv_i4 take: codes [tokens, heads, 64] and (scale, zero) pairs [tokens, heads, 2])
+__global__ __launch_bounds__(256) void kv_store_i4_kernel(const uint32_t *kq, const uint32_t *vq, const uint32_t *kpar,
+                                                          const uint32_t *vpar, const int32_t *seq_indptr, KvLayout c) {
+  const int b = blockIdx.x;
+  const int tok0 = seq_indptr ? seq_indptr[b] : b;
+  const int n_new = seq_indptr ? seq_indptr[b + 1] - tok0 : 1;
+  const int p0 = c.indptr[b], np = c.indptr[b + 1] - p0;
+  const int len = (np - 1) * c.page_size + c.last_page_offset[b];
+  const int lane16 = threadIdx.x & 15;
+  const int rows = n_new * c.heads;
+  for (int r = blockIdx.y * 16 + (threadIdx.x >> 4); r < rows; r += gridDim.y * 16) {
+    const int i = r / c.heads, head = r - i * c.heads;
+    const int pos = len - n_new + i;
+    const int page = c.indices[p0 + pos / c.page_size], slot = pos % c.page_size;
+    const size_t src = (size_t)(tok0 + i) * c.heads + head;
+    const size_t krow = kv_row(c, page, 0, head, slot), vrow = kv_row(c, page, 1, head, slot);
+    reinterpret_cast<uint32_t *>(c.data + krow * kRowBytes)[lane16] = kq[src * 16 + lane16];
+    reinterpret_cast<uint32_t *>(c.data + vrow * kRowBytes)[lane16] = vq[src * 16 + lane16];
+    if (lane16 == 0) {
+      c.param[krow] = kpar[src];
+      c.param[vrow] = vpar[src];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// decode: o[b, h] = softmax(q[b, h] . K[b]^T * sm_scale) V[b] for one new token per sequence.
+// One workgroup per (sequence, kv head); the G query heads of the group share every K / V read.
+// A row of 16 lanes covers the 128 dims of one token (4 code bytes = 8 dims per lane), so a wave
+// takes 4 tokens at a time and the workgroup 16.  With a stored value n standing for n*s - z,
+//   q . k = s * (q . n) - z * sum(q)     and     sum_t p_t v_t = sum_t (p_t s_t) n_t - sum_t p_t z_t,
+// so the codes are only converted to fp32, never dequantized element by element.
+// Each (wave, token slot) runs its own online softmax (base 2, sm_scale * log2(e) folded into q);
+// the 16 partial results are merged through LDS at the end.
+// ---------------------------------------------------------------------------------------------
+template <bool BF16, int G>
+__global__ __launch_bounds__(256) void kv_decode_i4_kernel(uint16_t *o, const uint16_t *q, KvLayout c, int num_qo_heads,
+                                                           float sm_scale_log2) {
+  __shared__ float part_o[16][G][kHeadDim];
+  __shared__ float part_ml[16][G][2];
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int dg = lane & 15, ts = lane >> 4;
+  const int p0 = c.indptr[b], np = c.indptr[b + 1] - p0;
+  const int len = np > 0 ? (np - 1) * c.page_size + c.last_page_offset[b] : 0;
+
+  float qv[G][8], qsum[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const uint4 raw = reinterpret_cast<const uint4 *>(q + ((size_t)b * num_qo_heads + h * G + g) * kHeadDim)[dg];
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      qv[g][2 * i] = from_bits<BF16>(w[i]) * sm_scale_log2;
+      qv[g][2 * i + 1] = from_bits<BF16>(w[i] >> 16) * sm_scale_log2;
+      s += qv[g][2 * i] + qv[g][2 * i + 1];
+    }
+    qsum[g] = row16_sum(s);
+  }
+
+  constexpr float kNegBig = -1e30f;
+  float m[G], l[G], zacc[G], acc[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = kNegBig;
+    l[g] = 0.0f;
+    zacc[g] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
+  }
+
+  for (int t0 = 0; t0 < len; t0 += 16) {
+    const int t = t0 + 4 * wave + ts;
+    const bool valid = t < len;
+    const int tc = valid ? t : len - 1;
+    const int page = c.indices[p0 + tc / c.page_size], slot = tc % c.page_size;
+    const size_t krow = kv_row(c, page, 0, h, slot), vrow = kv_row(c, page, 1, h, slot);
+    const uint32_t kd = reinterpret_cast<const uint32_t *>(c.data + krow * kRowBytes)[dg];
+    const uint32_t vd = reinterpret_cast<const uint32_t *>(c.data + vrow * kRowBytes)[dg];
+    const uint32_t kp = c.param[krow], vp = c.param[vrow];
+    const float ks = from_bits<BF16>(kp), kz = from_bits<BF16>(kp >> 16);
+    const float vs = from_bits<BF16>(vp), vz = from_bits<BF16>(vp >> 16);
+    float kn[8], vn[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      kn[i] = (float)((kd >> (4 * i)) & 15u);
+      vn[i] = (float)((vd >> (4 * i)) & 15u);
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float dot = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dot = __builtin_fmaf(qv[g][i], kn[i], dot);
+      dot = row16_sum(dot);
+      const float s = valid ? ks * dot - kz * qsum[g] : kNegBig;
+      const float mn = fmaxf(m[g], s);
+      const float corr = __builtin_amdgcn_exp2f(m[g] - mn);
+      const float p = __builtin_amdgcn_exp2f(s - mn);
+      m[g] = mn;
+      l[g] = l[g] * corr + p;
+      zacc[g] = zacc[g] * corr + p * vz;
+      const float pv = p * vs;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] = __builtin_fmaf(pv, vn[i], acc[g][i] * corr);
+    }
+  }
+
+  // merge the 16 partial softmaxes: part index = 4*wave + ts
+  const int pi = 4 * wave + ts;
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) part_o[pi][g][8 * dg + i] = acc[g][i] - zacc[g];
+    if (dg == 0) {
+      part_ml[pi][g][0] = m[g];
+      part_ml[pi][g][1] = l[g];
+    }
+  }
+  __syncthreads();
+  // thread -> (g, dim): G * 128 outputs over 256 threads
+  for (int idx = threadIdx.x; idx < G * kHeadDim; idx += 256) {
+    const int g = idx / kHeadDim, dim = idx - g * kHeadDim;
+    float M = kNegBig;
+#pragma unroll
+    for (int p = 0; p < 16; ++p) M = fmaxf(M, part_ml[p][g][0]);
+    float num = 0.0f, den = 0.0f;
+#pragma unroll
+    for (int p = 0; p < 16; ++p) {
+      const float wgt = __builtin_amdgcn_exp2f(part_ml[p][g][0] - M);
+      num = __builtin_fmaf(wgt, part_o[p][g][dim], num);
+      den = __builtin_fmaf(wgt, part_ml[p][g][1], den);
+    }
+    const float out = den > 0.0f ? num / den : 0.0f;
+    o[((size_t)b * num_qo_heads + h * G + g) * kHeadDim + dim] = (uint16_t)to_bits<BF16>(out);
+  }
+}
+
+int check_layout(const void *kv_data, const void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
+                 const int32_t *last_page_offset, int n_layers, int layer_idx, int heads, int page_size, int head_dim,
+                 int dtype) {
+  if (dtype != ARCQ_DTYPE_F16 && dtype != ARCQ_DTYPE_BF16) return ARCQ_ERR_FORMAT;
+  if (head_dim != kHeadDim || n_layers < 1 || layer_idx < 0 || layer_idx >= n_layers || heads < 1 || page_size < 1)
+    return ARCQ_ERR_SHAPE;
+  if (!kv_data || !kv_param || !kv_indptr || !kv_indices || !last_page_offset) return ARCQ_ERR_NULL;
+  if (!aligned16(kv_data) || ((uintptr_t)kv_param & 3)) return ARCQ_ERR_ALIGN;
+  return ARCQ_OK;
+}
+
+}  // namespace
+}  // namespace arcq
+
+extern "C" {
+
+int arcq_kv_append_i4(const void *k, const void *v, int dtype, int batch, const int32_t *seqlen_indptr, int max_new_tokens,
+                      void *kv_data, void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
+                      const int32_t *last_page_offset, int n_layers, int layer_idx, int num_kv_heads, int page_size,
+                      int head_dim, void *stream) {
+  using namespace arcq;
+  const int rc = check_layout(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, n_layers, layer_idx,
+                              num_kv_heads, page_size, head_dim, dtype);
+  if (rc != ARCQ_OK) return rc;
+  if (batch < 0 || max_new_tokens < 0) return ARCQ_ERR_SHAPE;
+  if (batch == 0 || max_new_tokens == 0) return ARCQ_OK;
+  if (!k || !v) return ARCQ_ERR_NULL;
+  if (!aligned16(k) || !aligned16(v)) return ARCQ_ERR_ALIGN;
+  KvLayout c{static_cast<uint8_t *>(kv_data), static_cast<uint32_t *>(kv_param), kv_indptr, kv_indices,
+             last_page_offset,               n_layers,                           layer_idx, num_kv_heads, page_size};
+  const long rows = (long)max_new_tokens * num_kv_heads;
+  int gy = (int)((rows + 15) / 16);
+  if (gy > 256) gy = 256;
+  dim3 grid(batch, gy);
+  if (dtype == ARCQ_DTYPE_BF16)
+    hipLaunchKernelGGL(kv_append_i4_kernel<true>, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t *>(k), static_cast<const uint16_t *>(v), seqlen_indptr, c);
+  else
+    hipLaunchKernelGGL(kv_append_i4_kernel<false>, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t *>(k), static_cast<const uint16_t *>(v), seqlen_indptr, c);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+int arcq_kv_store_i4(const void *k_codes, const void *v_codes, const void *k_param, const void *v_param, int batch,
+                     const int32_t *seqlen_indptr, int max_new_tokens, void *kv_data, void *kv_param,
+                     const int32_t *kv_indptr, const int32_t *kv_indices, const int32_t *last_page_offset, int n_layers,
+                     int layer_idx, int num_kv_heads, int page_size, int head_dim, void *stream) {
+  using namespace arcq;
+  const int rc = check_layout(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, n_layers, layer_idx,
+                              num_kv_heads, page_size, head_dim, ARCQ_DTYPE_F16);
+  if (rc != ARCQ_OK) return rc;
+  if (batch < 0 || max_new_tokens < 0) return ARCQ_ERR_SHAPE;
+  if (batch == 0 || max_new_tokens == 0) return ARCQ_OK;
+  if (!k_codes || !v_codes || !k_param || !v_param) return ARCQ_ERR_NULL;
+  if (((uintptr_t)k_codes | (uintptr_t)v_codes | (uintptr_t)k_param | (uintptr_t)v_param) & 3) return ARCQ_ERR_ALIGN;
+  KvLayout c{static_cast<uint8_t *>(kv_data), static_cast<uint32_t *>(kv_param), kv_indptr, kv_indices,
+             last_page_offset,               n_layers,                           layer_idx, num_kv_heads, page_size};
+  const long rows = (long)max_new_tokens * num_kv_heads;
+  int gy = (int)((rows + 15) / 16);
+  if (gy > 256) gy = 256;
+  hipLaunchKernelGGL(kv_store_i4_kernel, dim3(batch, gy), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint32_t *>(k_codes), static_cast<const uint32_t *>(v_codes),
+                     static_cast<const uint32_t *>(k_param), static_cast<const uint32_t *>(v_param), seqlen_indptr, c);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+int arcq_kv_decode_i4(void *o, const void *q, int dtype, int batch, int num_qo_heads, const void *kv_data,
+                      const void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
+                      const int32_t *last_page_offset, int n_layers, int layer_idx, int num_kv_heads, int page_size,
+                      int head_dim, float sm_scale, void *stream) {
+  using namespace arcq;
+  const int rc = check_layout(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, n_layers, layer_idx,
+                              num_kv_heads, page_size, head_dim, dtype);
+  if (rc != ARCQ_OK) return rc;
+  if (batch < 0 || num_qo_heads < num_kv_heads || num_qo_heads % num_kv_heads != 0) return ARCQ_ERR_SHAPE;
+  const int G = num_qo_heads / num_kv_heads;
+  if (G != 1 && G != 2 && G != 4) return ARCQ_ERR_SHAPE;  // query heads per KV head
+  if (batch == 0) return ARCQ_OK;
+  if (!o || !q) return ARCQ_ERR_NULL;
+  if (!aligned16(o) || !aligned16(q)) return ARCQ_ERR_ALIGN;
+  KvLayout c{const_cast<uint8_t *>(static_cast<const uint8_t *>(kv_data)),
+             const_cast<uint32_t *>(static_cast<const uint32_t *>(kv_param)),
+             kv_indptr,
+             kv_indices,
+             last_page_offset,
+             n_layers,
+             layer_idx,
+             num_kv_heads,
+             page_size};
+  const float sl2 = sm_scale * 1.4426950408889634f;
+  dim3 grid(batch, num_kv_heads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint16_t *op = static_cast<uint16_t *>(o);
+  const uint16_t *qp = static_cast<const uint16_t *>(q);
+#define ARCQ_LAUNCH_DECODE(BF, GG) \
+  hipLaunchKernelGGL((kv_decode_i4_kernel<BF, GG>), grid, dim3(256), 0, st, op, qp, c, num_qo_heads, sl2)
+  if (dtype == ARCQ_DTYPE_BF16) {
+    if (G == 1) ARCQ_LAUNCH_DECODE(true, 1);
+    else if (G == 2) ARCQ_LAUNCH_DECODE(true, 2);
+    else ARCQ_LAUNCH_DECODE(true, 4);
+  } else {
+    if (G == 1) ARCQ_LAUNCH_DECODE(false, 1);
+    else if (G == 2) ARCQ_LAUNCH_DECODE(false, 2);
+    else ARCQ_LAUNCH_DECODE(false, 4);
+  }
+#undef ARCQ_LAUNCH_DECODE
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+}  // extern "C"

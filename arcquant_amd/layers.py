@@ -216,9 +216,11 @@ class LlamaAttention(nn.Module):
         self.quant_type = quant_type
 
     @torch.no_grad()
-    def forward(self, x, kv_cache=None, past_len=0):
-        """x: quantized hidden states (tuple).  kv_cache: None or (k, v) bf16 [bsz, kv_heads, L, d]
-        holding past_len valid positions; the new keys/values are written behind them."""
+    def forward(self, x, kv_cache=None, past_len=0, layer_idx=0):
+        """x: quantized hidden states (tuple).  kv_cache: None, or (k, v) bf16 [bsz, kv_heads, L, d]
+        holding past_len valid positions (the new keys/values are written behind them), or an
+        arcquant_amd.kv_cache.MultiLayerPagedKVCache4Bit (INT4 pages; decode attention then runs on
+        the quantized cache, model/qLlamaLayer.py:334-338 with model/kv_cache.py:214-279)."""
         bsz, q_len = x[3], x[4]
         d, nh, nkv = self.head_dim, self.num_heads, self.num_kv_heads
         qkv = self.qkv_proj(x)
@@ -226,6 +228,13 @@ class LlamaAttention(nn.Module):
         k = qkv[..., nh * d:(nh + nkv) * d].view(bsz, q_len, nkv, d).transpose(1, 2)
         v = qkv[..., (nh + nkv) * d:].view(bsz, q_len, nkv, d).transpose(1, 2)
         q, k = rotary_pos_emb(q, k, past_len)
+        if kv_cache is not None and not isinstance(kv_cache, tuple):
+            r = kv_cache.update(k.transpose(1, 2), v.transpose(1, 2), layer_idx)
+            if callable(r):                                   # decode: attention over the INT4 pages
+                out = r(q.transpose(1, 2)).reshape(bsz, q_len, nh * d)
+                return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num,
+                                                   self.quant_type))
+            kv_cache = None                                   # prefill: attend to the fresh keys / values
         if kv_cache is not None:
             kc, vc = kv_cache
             kc[:, :, past_len:past_len + q_len] = k
@@ -268,8 +277,8 @@ class LlamaDecoderLayer(nn.Module):
                             down_idx, quant_type)
 
     @torch.no_grad()
-    def forward(self, hidden_states, kv_cache=None, past_len=0):
-        h = hidden_states + self.self_attn(self.input_layernorm(hidden_states), kv_cache, past_len)
+    def forward(self, hidden_states, kv_cache=None, past_len=0, layer_idx=0):
+        h = hidden_states + self.self_attn(self.input_layernorm(hidden_states), kv_cache, past_len, layer_idx)
         return h + self.mlp(self.post_attention_layernorm(h))
 
 

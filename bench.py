@@ -224,7 +224,21 @@ def layer_rows(torch, iters=10):
                      "arc_ms": round(ms_arc, 3), "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_arc, 2),
                      "tokens_per_s": round(64 / ms_arc * 1e3)})
         print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
-        del layer, W, kv, x
+        # the same decode step over an INT4 paged KV cache (decode attention on the quantized pages)
+        from arcquant_amd.kv_cache import MultiLayerPagedKVCache4Bit
+        cache = MultiLayerPagedKVCache4Bit(64, 16, kvlen + 64, "cuda", 1, nkv, d, dtype=torch.bfloat16)
+        cache.update(kv[0][:, :, :kvlen].transpose(1, 2).contiguous(), kv[1][:, :, :kvlen].transpose(1, 2).contiguous(), 0)
+
+        def paged_step():
+            cache.lengths = [kvlen] * 64          # keep the length fixed across timed repetitions
+            cache._specs["last_page_offset"].fill_(kvlen % 16 or 16)
+            return layer(x, cache, kvlen)
+        ms_i4 = timed(paged_step)
+        rows.append({"config": f"decoder layer decode batch 64, KV length {kvlen}, INT4 paged KV cache", "fmt": fmt,
+                     "arc_ms": round(ms_i4, 3), "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_i4, 2),
+                     "tokens_per_s": round(64 / ms_i4 * 1e3)})
+        print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
+        del layer, W, kv, x, cache
         torch.cuda.empty_cache()
 
     # Mixtral block, NVFP4 (benchmark configuration 5), select_num 128

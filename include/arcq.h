@@ -136,6 +136,46 @@ int arcq_matmul(const void *a_codes, const void *a_scales, const void *b_codes, 
                 void *stream);
 
 /*
+ * INT4 paged KV cache (the reference's decode-attention path: agemm.init_kv_i4 / append_kv_i4 /
+ * batch_decode_i4, kernels/src/bindings.cpp:287-413 -> kernels/src/flashinfer.cu:9-112, with the
+ * torch-side quantizer asym_quantize_and_pack_i4, model/kv_cache.py:23-37, fused into the append).
+ * Container layout as the reference allocates it (model/kv_cache.py:148-160):
+ *   kv_data   u8 [pages, n_layers, 2 (k, v), kv_heads, page_size, head_dim/2], element 2j in the low nibble
+ *   kv_param  [pages, n_layers, 2, kv_heads, page_size, 2] = (scale, zero) per (token, head) in `dtype`;
+ *             a stored n stands for n * scale - zero (model/kv_cache.py:39-43)
+ *   kv_indptr int32 [batch+1], kv_indices int32, last_page_offset int32 [batch]: sequence b owns pages
+ *             kv_indices[kv_indptr[b] .. kv_indptr[b+1]) and holds (pages_b - 1) * page_size +
+ *             last_page_offset[b] tokens
+ * dtype: ARCQ_DTYPE_F16 (the reference's) or ARCQ_DTYPE_BF16, for k, v, q, o and kv_param alike.
+ * head_dim must be 128 (flashinfer.cu:212-223 instantiates nothing else).
+ *
+ * arcq_kv_append_i4 quantizes new keys / values [tokens, kv_heads, 128] and writes them into their
+ * pages; the page table describes the state AFTER the append (as model/kv_cache.py:228-262 passes it).
+ *   seqlen_indptr  int32 [batch+1] offsets of each sequence's new tokens in k / v (prefill,
+ *                  replaces init_kv_i4), or NULL for one new token per sequence (append_kv_i4)
+ *   max_new_tokens upper bound of new tokens per sequence (sizes the launch)
+ * arcq_kv_decode_i4: o[b, h, :] = softmax(q[b, h] . K_b^T * sm_scale) V_b over the dequantized cache, one
+ * query token per sequence; q, o [batch, num_qo_heads, 128]; num_qo_heads / num_kv_heads in {1, 2, 4}
+ * (the reference's kernel takes equal head counts only).  fp32 softmax and accumulation.
+ */
+enum { ARCQ_DTYPE_F16 = 0, ARCQ_DTYPE_BF16 = 1 };
+int arcq_kv_append_i4(const void *k, const void *v, int dtype, int batch, const int32_t *seqlen_indptr, int max_new_tokens,
+                      void *kv_data, void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
+                      const int32_t *last_page_offset, int n_layers, int layer_idx, int num_kv_heads, int page_size,
+                      int head_dim, void *stream);
+/* the same scatter for rows the caller has quantized already -- the exact argument set of the
+ * reference's init_kv_i4 (seqlen_indptr given) and append_kv_i4 (seqlen_indptr NULL):
+ * k_codes / v_codes u8 [tokens, kv_heads, 64], k_param / v_param [tokens, kv_heads, 2] */
+int arcq_kv_store_i4(const void *k_codes, const void *v_codes, const void *k_param, const void *v_param, int batch,
+                     const int32_t *seqlen_indptr, int max_new_tokens, void *kv_data, void *kv_param,
+                     const int32_t *kv_indptr, const int32_t *kv_indices, const int32_t *last_page_offset, int n_layers,
+                     int layer_idx, int num_kv_heads, int page_size, int head_dim, void *stream);
+int arcq_kv_decode_i4(void *o, const void *q, int dtype, int batch, int num_qo_heads, const void *kv_data,
+                      const void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
+                      const int32_t *last_page_offset, int n_layers, int layer_idx, int num_kv_heads, int page_size,
+                      int head_dim, float sm_scale, void *stream);
+
+/*
  * Debug helper: checks on the device that reorder_index is a permutation of 0..K-1 and
  * returns ARCQ_ERR_INDEX otherwise.  Synchronises `stream`.  The reference performs no such
  * check (kernels/src/reorder.cu:117 indexes shared memory with whatever it is given).

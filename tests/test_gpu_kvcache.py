@@ -1,0 +1,164 @@
+"""INT4 paged KV cache on the GPU: the fused quantize + append against the torch restatement of
+model/kv_cache.py:23-37 (codes and (scale, zero) pairs bit-exact), the pre-quantized store, and the
+decode attention against fp64 softmax attention over the dequantized cache.  Attention tolerance:
+relative Frobenius error of the fp16 / bf16 output <= 1e-3 / 5e-3 (the output rounding alone is
+3e-4 / 2e-3; the kernel accumulates in fp32)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float16, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def kvc():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from arcquant_amd import kv_cache as m
+    return m
+
+
+@pytest.fixture(scope="module")
+def ref():
+    from oracle import kvcache_torch as m
+    return m
+
+
+def make_table(lengths, page_size, batch):
+    """pages of sequence b: b, b + batch, ... (model/kv_cache.py:293-296)"""
+    cnt = [(n + page_size - 1) // page_size for n in lengths]
+    indptr, indices, last = [0], [], []
+    for b, (n, c) in enumerate(zip(lengths, cnt)):
+        indptr.append(indptr[-1] + c)
+        indices += [j * batch + b for j in range(c)]
+        off = n % page_size
+        last.append(page_size if (n and off == 0) else off)
+    t = lambda x: torch.tensor(x, dtype=torch.int32)
+    return t(indptr), t(indices), t(last), max(cnt) if cnt else 0
+
+
+def rel_fro(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return float((got - want).norm() / want.norm())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_quantize_append_is_bit_exact(kvc, ref, dtype):
+    batch, heads, page_size, layers, layer = 3, 2, 16, 2, 1
+    lengths = [37, 16, 5]                                   # ragged prefill, page boundary, short
+    g = torch.Generator().manual_seed(3)
+    total = sum(lengths)
+    k = (torch.randn(total, heads, 128, generator=g) * 2).to(dtype)
+    v = torch.randn(total, heads, 128, generator=g).to(dtype)
+    k[3] = 0.25                                             # constant row: max - min below the clamp
+    v[4, 0, :64] = 0
+    indptr, indices, last, maxc = make_table(lengths, page_size, batch)
+    pages = torch.zeros((maxc + 1) * batch, layers, 2, heads, page_size, 64, dtype=torch.uint8, device="cuda")
+    params = torch.zeros((maxc + 1) * batch, layers, 2, heads, page_size, 2, dtype=dtype, device="cuda")
+    seq = torch.tensor([0, 37, 53, 58], dtype=torch.int32)
+    print(f"kv append {dtype}", flush=True)
+    kvc.quantize_append(pages, params, indptr.cuda(), indices.cuda(), last.cuda(), k.cuda(), v.cuda(), layer,
+                        seqlen_indptr=seq.cuda())
+    # one more token per sequence (crosses a page boundary for sequence 1: 16 -> 17)
+    lengths2 = [n + 1 for n in lengths]
+    indptr2, indices2, last2, _ = make_table(lengths2, page_size, batch)
+    k1 = torch.randn(batch, heads, 128, generator=g).to(dtype)
+    v1 = torch.randn(batch, heads, 128, generator=g).to(dtype)
+    kvc.quantize_append(pages, params, indptr2.cuda(), indices2.cuda(), last2.cuda(), k1.cuda(), v1.cuda(), layer)
+
+    pc, sc = pages.cpu(), params.cpu()
+    assert int(pc[:, 0].sum()) == 0 and float(sc[:, 0].abs().sum()) == 0          # the other layer is untouched
+    for b in range(batch):
+        (kc, kp), (vc, vp) = ref.gather_sequence(pc, sc, indptr2, indices2, last2, layer, b)
+        lo = int(seq[b])
+        kb = torch.cat([k[lo:lo + lengths[b]], k1[b:b + 1]])
+        vb = torch.cat([v[lo:lo + lengths[b]], v1[b:b + 1]])
+        for codes, par, x in ((kc, kp, kb), (vc, vp, vb)):
+            q, s, z = ref.asym_quantize_and_pack_i4(x)
+            assert torch.equal(codes, ref.unpack(q))
+            assert torch.equal(par[..., 0], s[..., 0].double()) and torch.equal(par[..., 1], z[..., 0].double())
+
+
+def test_store_prequantized_rows(kvc, ref):
+    batch, heads, page_size = 2, 4, 8
+    lengths = [9, 8]
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(sum(lengths), heads, 128, generator=g).half()
+    kq, ks, kz = ref.asym_quantize_and_pack_i4(x)
+    vq, vs, vz = ref.asym_quantize_and_pack_i4(-x)
+    kp, vp = torch.cat([ks, kz], -1), torch.cat([vs, vz], -1)
+    indptr, indices, last, maxc = make_table(lengths, page_size, batch)
+    pages = torch.zeros(maxc * batch, 1, 2, heads, page_size, 64, dtype=torch.uint8, device="cuda")
+    params = torch.zeros(maxc * batch, 1, 2, heads, page_size, 2, dtype=torch.float16, device="cuda")
+    seq = torch.tensor([0, 9, 17], dtype=torch.int32).cuda()
+    kvc.init_kv_i4(pages, params, indptr.cuda(), indices.cuda(), last.cuda(), kq.cuda(), vq.cuda(), kp.cuda(), vp.cuda(),
+                   seq, 0)
+    for b, lo in enumerate((0, 9)):
+        (kc, kpar), (vc, vpar) = ref.gather_sequence(pages.cpu(), params.cpu(), indptr, indices, last, 0, b)
+        assert torch.equal(kc, ref.unpack(kq[lo:lo + lengths[b]]))
+        assert torch.equal(vc, ref.unpack(vq[lo:lo + lengths[b]]))
+        assert torch.equal(kpar, kp[lo:lo + lengths[b]].double()) and torch.equal(vpar, vp[lo:lo + lengths[b]].double())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("q_heads,kv_heads", [(4, 4), (8, 4), (32, 8)])
+def test_decode_attention(kvc, ref, dtype, q_heads, kv_heads):
+    batch, page_size, layers, layer = 4, 16, 2, 0
+    lengths = [1, 16, 77, 260]
+    g = torch.Generator().manual_seed(5)
+    total = sum(lengths)
+    k = (torch.randn(total, kv_heads, 128, generator=g) * 1.5).to(dtype)
+    v = torch.randn(total, kv_heads, 128, generator=g).to(dtype)
+    q = torch.randn(batch, q_heads, 128, generator=g).to(dtype)
+    indptr, indices, last, maxc = make_table(lengths, page_size, batch)
+    pages = torch.zeros(maxc * batch, layers, 2, kv_heads, page_size, 64, dtype=torch.uint8, device="cuda")
+    params = torch.zeros(maxc * batch, layers, 2, kv_heads, page_size, 2, dtype=dtype, device="cuda")
+    offs = [0]
+    for n in lengths:
+        offs.append(offs[-1] + n)
+    print(f"kv decode {dtype} heads {q_heads}/{kv_heads}", flush=True)
+    kvc.quantize_append(pages, params, indptr.cuda(), indices.cuda(), last.cuda(), k.cuda(), v.cuda(), layer,
+                        seqlen_indptr=torch.tensor(offs, dtype=torch.int32).cuda())
+    o = torch.empty_like(q).cuda()
+    kvc.batch_decode_i4(o, q.cuda(), pages, params, indptr.cuda(), indices.cuda(), last.cuda(), layer)
+    want = ref.decode_attention(q, pages.cpu(), params.cpu(), indptr, indices, last, layer)
+    tol = 1e-3 if dtype == torch.float16 else 5e-3
+    assert rel_fro(o, want) < tol
+    # a one-token sequence returns that token's dequantized value row
+    (kc, kp), (vc, vp) = ref.gather_sequence(pages.cpu(), params.cpu(), indptr, indices, last, layer, 0)
+    v0 = vc.double() * vp[..., :1] - vp[..., 1:]
+    assert rel_fro(o[0, 0], v0[0, 0]) < tol
+
+
+def test_cache_container_flow(kvc, ref):
+    """prefill + three decode steps through MultiLayerPagedKVCache4Bit on two layers"""
+    batch, heads, q_heads, layers, page_size = 2, 2, 4, 2, 16
+    dtype = torch.bfloat16
+    cache = kvc.MultiLayerPagedKVCache4Bit(batch, page_size, 64, "cuda", layers, heads, 128, dtype=dtype)
+    g = torch.Generator().manual_seed(6)
+    hist = {l: [] for l in range(layers)}
+    for step, t in enumerate((30, 1, 1, 1)):
+        for l in range(layers):
+            k = torch.randn(batch, t, heads, 128, generator=g).to(dtype)
+            v = torch.randn(batch, t, heads, 128, generator=g).to(dtype)
+            hist[l].append((k, v))
+            r = cache.update(k.cuda(), v.cuda(), l)
+            if step == 0:
+                assert isinstance(r, tuple)
+                continue
+            q = torch.randn(batch, 1, q_heads, 128, generator=g).to(dtype)
+            out = r(q.cuda())
+            assert out.shape == (batch, 1, q_heads, 128)
+            kall = torch.cat([a for a, _ in hist[l]], dim=1)
+            vall = torch.cat([b for _, b in hist[l]], dim=1)
+            kq, ks, kz = ref.asym_quantize_and_pack_i4(kall)
+            vq, vs, vz = ref.asym_quantize_and_pack_i4(vall)
+            kd = ref.unpack(kq).double() * ks.double() - kz.double()
+            vd = ref.unpack(vq).double() * vs.double() - vz.double()
+            gsz = q_heads // heads
+            want = torch.zeros(batch, q_heads, 128, dtype=torch.float64)
+            for b in range(batch):
+                for h in range(q_heads):
+                    s = (kd[b, :, h // gsz] @ q[b, 0, h].double()) * 128 ** -0.5
+                    want[b, h] = torch.softmax(s, 0) @ vd[b, :, h // gsz]
+            assert rel_fro(out[:, 0], want) < 5e-3
+    assert cache.get_seq_length() == 33
