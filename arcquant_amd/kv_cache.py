@@ -146,13 +146,20 @@ class MultiLayerPagedKVCache4Bit:
         self.batch_size, self.page_size, self.max_seq_len = batch_size, page_size, max_seq_len
         self.device, self.n_layers, self.num_heads, self.head_dim = device, n_layers, num_heads, head_dim
         max_page_cnt = self.page_cnt_from_length(max_seq_len)
-        self.pages = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, head_dim // 2),
+        self.pages = torch.zeros((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, head_dim // 2),
                                  dtype=torch.uint8, device=device)
-        self.scales = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, 2), dtype=dtype,
+        self.scales = torch.zeros((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, 2), dtype=dtype,
                                   device=device)
         self._needs_init = [True] * n_layers
         self.lengths = [0] * batch_size          # host mirror of the sequence lengths
+        # The page table lives in tensors allocated once and updated in place, so that a captured HIP
+        # graph of a decode step keeps reading the right addresses.  `positions` holds the position of
+        # each sequence's newest token (for rotary embeddings inside a graph).
+        mk = lambda n: torch.zeros(n, dtype=torch.int32, device=device)
+        self._indptr, self._indices, self._last = mk(batch_size + 1), mk(max(1, max_page_cnt * batch_size)), mk(batch_size)
+        self.positions = mk(batch_size)
         self._specs = None
+        self.external_step = False                # True: the caller advances the cache with begin_step()
 
     def page_cnt_from_length(self, length):
         return (length + self.page_size - 1) // self.page_size
@@ -183,9 +190,13 @@ class MultiLayerPagedKVCache4Bit:
         indices = grid[np.arange(maxc)[None, :] < cnt[:, None]].astype(np.int32)
         off = lens % ps
         last = np.where((lens != 0) & (off == 0), ps, off).astype(np.int32)
-        mk = lambda a: torch.from_numpy(a if a.size else np.zeros(1, np.int32)).to(self.device)
-        self._specs = {"kv_data": self.pages, "kv_param": self.scales, "kv_indptr": mk(indptr),
-                       "kv_indices": mk(indices), "last_page_offset": mk(last)}
+        self._indptr.copy_(torch.from_numpy(indptr))
+        if indices.size:
+            self._indices[:indices.size].copy_(torch.from_numpy(indices))
+        self._last.copy_(torch.from_numpy(last))
+        self.positions.copy_(torch.from_numpy(np.maximum(lens - 1, 0).astype(np.int32)))
+        self._specs = {"kv_data": self.pages, "kv_param": self.scales, "kv_indptr": self._indptr,
+                       "kv_indices": self._indices, "last_page_offset": self._last}
         return self._specs
 
     def _advance_one_token(self):
@@ -197,7 +208,14 @@ class MultiLayerPagedKVCache4Bit:
         if new_page or self._specs is None:
             self._build_specs()
         else:
-            self._specs["last_page_offset"].add_(1)
+            self._last.add_(1)
+            self.positions.add_(1)
+
+    def begin_step(self):
+        """Advance every sequence by one token ahead of a decode step whose launches are replayed from
+        a captured graph: the host-side bookkeeping happens here, the graph only launches kernels.
+        Use with external_step = True."""
+        self._advance_one_token()
 
     def get_cache_specs_for_flash_infer(self, attention_mask=None):
         return self._specs if self._specs is not None else self._build_specs()
@@ -229,7 +247,7 @@ class MultiLayerPagedKVCache4Bit:
                             max_new_tokens=max(new), **self._specs)
             return key_states, value_states
         assert added == 1
-        if layer_idx == 0:
+        if layer_idx == 0 and not self.external_step:
             self._advance_one_token()
         quantize_append(k=key_states.reshape(b_sz, heads, head_dim).contiguous(),
                         v=value_states.reshape(b_sz, heads, head_dim).contiguous(), layer_idx=layer_idx, **self._specs)

@@ -160,12 +160,19 @@ def _rotate_half(x):
 
 
 def rotary_pos_emb(q, k, beg, base=10000.0):
-    """benchmarks/modeling_arc.py:63-78: rotary embedding for positions beg .. beg+seqlen."""
+    """benchmarks/modeling_arc.py:63-78: rotary embedding for positions beg .. beg+seqlen.
+    beg may also be an int32 tensor [batch] of per-sequence positions (one new token each), read on the
+    device -- what a decode step replayed from a captured graph needs."""
     dim, seqlen = q.shape[-1], q.shape[-2]
     inv_freq = 1.0 / (base ** (torch.arange(0, dim, 2, device=q.device).float() / dim))
-    t = torch.arange(beg, beg + seqlen, device=q.device, dtype=torch.float32)
-    freqs = torch.outer(t, inv_freq)
-    emb = torch.cat((freqs, freqs), dim=-1)[None, None]
+    if isinstance(beg, torch.Tensor):
+        t = beg.to(torch.float32)[:, None] + torch.arange(seqlen, device=q.device, dtype=torch.float32)[None, :]
+        freqs = t[:, :, None] * inv_freq[None, None, :]                     # [batch, seqlen, dim/2]
+        emb = torch.cat((freqs, freqs), dim=-1)[:, None]                    # [batch, 1, seqlen, dim]
+    else:
+        t = torch.arange(beg, beg + seqlen, device=q.device, dtype=torch.float32)
+        freqs = torch.outer(t, inv_freq)
+        emb = torch.cat((freqs, freqs), dim=-1)[None, None]
     cos, sin = emb.cos().to(q.dtype), emb.sin().to(q.dtype)
     return q * cos + _rotate_half(q) * sin, k * cos + _rotate_half(k) * sin
 
@@ -362,3 +369,44 @@ def build_mixtral_block(hidden=4096, ffn=14336, num_experts=8, top_k=2, select_n
         experts.append(MixtralExpertMLP(w1, w3, w2, select_num, i_in, i_w2, quant_type))
         del w1, w3, w2
     return MixtralSparseMoeBlock(gate, experts, top_k)
+
+
+class GraphedDecodeStep:
+    """One decoder layer's decode step (one new token per sequence, INT4 paged KV cache) captured
+    once as a HIP graph and replayed: the step is a chain of ~60 short launches whose issue cost on
+    the host exceeds their run time.  Host-side cache bookkeeping happens in cache.begin_step() before
+    each replay; the token positions for the rotary embedding are read from cache.positions on the
+    device.  No memset nodes are recorded (buffers are cleared by fill kernels)."""
+
+    def __init__(self, layer: LlamaDecoderLayer, cache, batch, hidden, layer_idx=0, warmup=3):
+        self.layer, self.cache, self.layer_idx = layer, cache, layer_idx
+        cache.external_step = True
+        self.x = torch.zeros(batch, 1, hidden, dtype=torch.bfloat16, device=cache.device)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        saved = list(cache.lengths)
+        with torch.cuda.stream(side):            # warm-up on a side stream, as graph capture requires
+            for _ in range(warmup):
+                cache.begin_step()
+                self._run()
+                self._rewind(saved)
+        torch.cuda.current_stream().wait_stream(side)
+        cache.begin_step()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.y = self._run()
+        self._rewind(saved)
+
+    def _rewind(self, lengths):
+        self.cache.lengths = list(lengths)
+        self.cache._build_specs()
+
+    def _run(self):
+        return self.layer(self.x, self.cache, self.cache.positions, self.layer_idx)
+
+    @torch.no_grad()
+    def __call__(self, hidden_states):
+        self.cache.begin_step()
+        self.x.copy_(hidden_states)
+        self.graph.replay()
+        return self.y

@@ -238,7 +238,17 @@ def layer_rows(torch, iters=10):
                      "arc_ms": round(ms_i4, 3), "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_i4, 2),
                      "tokens_per_s": round(64 / ms_i4 * 1e3)})
         print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
-        del layer, W, kv, x, cache
+        # ... and the whole step replayed from a captured HIP graph (the KV length grows by one per
+        # replay, as in generation: 2048 -> ~2060 over the timed repetitions)
+        cache2 = MultiLayerPagedKVCache4Bit(64, 16, kvlen + 256, "cuda", 1, nkv, d, dtype=torch.bfloat16)
+        cache2.update(kv[0][:, :, :kvlen].transpose(1, 2).contiguous(), kv[1][:, :, :kvlen].transpose(1, 2).contiguous(), 0)
+        step = layers.GraphedDecodeStep(layer, cache2, 64, hidden)
+        ms_g = timed(lambda: step(x))
+        rows.append({"config": f"decoder layer decode batch 64, KV length {kvlen}+, INT4 paged KV cache, HIP graph",
+                     "fmt": fmt, "arc_ms": round(ms_g, 3), "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_g, 2),
+                     "tokens_per_s": round(64 / ms_g * 1e3)})
+        print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
+        del layer, W, kv, x, cache, cache2, step
         torch.cuda.empty_cache()
 
     # Mixtral block, NVFP4 (benchmark configuration 5), select_num 128

@@ -167,3 +167,31 @@ def test_mixtral_block_matches_reference_loop(layers, fq, fmt):
         want.index_add_(0, top_x, out * w[top_x, slot, None])
     assert rel_fro(y.view(tokens, hidden), want) < 2e-2
     assert float(y.abs().sum()) > 0
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_graphed_decode_step_matches_eager(layers, fmt):
+    """A decode step over the INT4 paged KV cache replayed from a captured HIP graph gives what the
+    eager step gives, on every replay, with eager work and synchronisation between replays, across a
+    page boundary (page size 16, lengths 14 -> 19)."""
+    from arcquant_amd.kv_cache import MultiLayerPagedKVCache4Bit
+    hidden, inter, nh, nkv, S, batch, page = 512, 1024, 4, 2, 64, 3, 16
+    layer = layers.LlamaDecoderLayer(hidden, inter, nh, nkv, select_num=S, select_num_down=S, quant_type=fmt, seed=12)
+    g = torch.Generator().manual_seed(13)
+    prompt = torch.randn(batch, 14, hidden, generator=g).to(torch.bfloat16).cuda()
+    caches = [MultiLayerPagedKVCache4Bit(batch, page, 64, "cuda", 1, nkv, 128, dtype=torch.bfloat16) for _ in range(2)]
+    for c in caches:
+        layer(prompt, c, 0)
+    eager_cache, graph_cache = caches
+    step = layers.GraphedDecodeStep(layer, graph_cache, batch, hidden)
+    assert graph_cache.lengths == [14] * batch                      # capture left the cache where it was
+    for i in range(5):
+        x = torch.randn(batch, 1, hidden, generator=g).to(torch.bfloat16).cuda()
+        print(f"graphed decode {fmt} step {i}", flush=True)
+        want = layer(x, eager_cache, eager_cache.lengths[0])        # eager: position = current length
+        torch.cuda.synchronize()
+        got = step(x).clone()
+        torch.cuda.synchronize()
+        assert graph_cache.lengths == eager_cache.lengths
+        assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
+    assert torch.equal(graph_cache.pages, eager_cache.pages) and torch.equal(graph_cache.scales, eager_cache.scales)
