@@ -16,6 +16,7 @@
 // head_dim is 128 (the only instantiation of the reference, flashinfer.cu:212-223).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "../../include/arcq.h"
 #include "arcq_internal.h"
@@ -273,6 +274,204 @@ __global__ __launch_bounds__(256) void kv_decode_i4_kernel(uint16_t *o, const ui
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same decode on the matrix cores, for page sizes that are multiples of 16.  A wave takes chunks
+// of 16 tokens (always inside one page):
+//   S^T[token, head] = Kn[token, dim] . Q^T[dim, head]      4 x v_mfma_f32_16x16x32_f16
+//   O[head, dim]    += P[head, token] . Vn[token, dim]      8 x v_mfma_f32_16x16x16_f16
+// Kn, Vn are the stored codes 0..15 as fp16; scale and zero of the rows enter through the identities
+// above (s * dot - z * sum(q), and p * s_v folded into P), so no element is dequantized.
+// Codes become fp16 by or-ing them into the mantissa of 1024 (0x6400 | n = 1024 + n; the high nibble
+// of a byte lands four bits up and reads 1024 + 16 n): for K the 1024 is subtracted exactly with a
+// packed add and the factor 16 is divided out of the matching q elements; for V both are removed
+// from the accumulated sums at the end (sum_t p_t * 1024 is tracked beside the softmax denominator).
+// Layouts make every operand a plain load: the K operand row of a lane is its token's 16 bytes
+// (the MFMA's K index is a permutation of the dims, applied to Q^T as well), S^T comes out with a
+// lane holding 4 tokens of one head, which is exactly the A operand of the second product, and the
+// V operand of a lane is one dword (8 dims) of each of its 4 tokens, output column j of MFMA j being
+// dim 8 * (lane % 16) + j.
+// ---------------------------------------------------------------------------------------------
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+
+// byte I of x into the low byte of both halves of a dword
+template <int I>
+__device__ __forceinline__ uint32_t spread_byte(uint32_t x) {
+  return __builtin_amdgcn_perm(0u, x, 0x0c000c00u | ((uint32_t)I << 16) | (uint32_t)I);
+}
+// (lo nibble, hi nibble * 16) of the spread byte as fp16, 1024 removed
+__device__ __forceinline__ uint32_t nibbles_exact(uint32_t t) {
+  typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+  const v2h v = __builtin_bit_cast(v2h, (t & 0x00f0000fu) | 0x64006400u);
+  const v2h off = {(_Float16)1024.0f, (_Float16)1024.0f};
+  return __builtin_bit_cast(uint32_t, v - off);
+}
+__device__ __forceinline__ v8h k_operand(uint32_t x) {  // 8 codes -> (n0, 16 n1, n2, 16 n3, ...)
+  v4u d;
+  d[0] = nibbles_exact(spread_byte<0>(x));
+  d[1] = nibbles_exact(spread_byte<1>(x));
+  d[2] = nibbles_exact(spread_byte<2>(x));
+  d[3] = nibbles_exact(spread_byte<3>(x));
+  return __builtin_bit_cast(v8h, d);
+}
+
+template <bool BF16, int G>
+__global__ __launch_bounds__(256) void kv_decode_i4_mfma_kernel(uint16_t *o, const uint16_t *q, KvLayout c,
+                                                                int num_qo_heads, float sm_scale_log2) {
+  __shared__ float part_o[4][G][kHeadDim];
+  __shared__ float part_s[4][G][4];  // m, l, D (1024 * sum of P), Z (sum of p * zero)
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int p0 = c.indptr[b], np = c.indptr[b + 1] - p0;
+  const int len = np > 0 ? (np - 1) * c.page_size + c.last_page_offset[b] : 0;
+  constexpr float kNegBig = -1e30f;
+
+  // Q^T operand: lane (head r16, group g) holds dims 32g + 8m + e for MFMA m, odd e divided by 16
+  v8h qop[4];
+  float qsum = 0.0f;
+  {
+    const bool real = r16 < G;
+    const uint16_t *qrow = q + ((size_t)b * num_qo_heads + h * G + (real ? r16 : 0)) * kHeadDim + 32 * g;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const uint4 raw = reinterpret_cast<const uint4 *>(qrow)[m];
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float f = from_bits<BF16>(w[e >> 1] >> (16 * (e & 1)));
+        if (!real) f = 0.0f;
+        const _Float16 hq = (_Float16)f;                 // exact for bf16 inputs inside the fp16 range
+        qsum += (float)hq;
+        qop[m][e] = (e & 1) ? hq * (_Float16)0.0625f : hq;
+      }
+    }
+    qsum += __shfl_xor(qsum, 16);
+    qsum += __shfl_xor(qsum, 32);
+  }
+
+  float m_run = kNegBig, l_run = 0.0f, d_run = 0.0f, z_run = 0.0f;
+  v4f oacc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) oacc[j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  const int nchunks = (len + 15) >> 4;
+  for (int ch = wave; ch < nchunks; ch += 4) {
+    const int t0 = ch << 4;
+    const int page = c.indices[p0 + t0 / c.page_size], slot0 = t0 % c.page_size;
+    const size_t krow0 = kv_row(c, page, 0, h, slot0), vrow0 = kv_row(c, page, 1, h, slot0);
+    // K: this lane's token r16, bytes 16g .. 16g+15
+    const uint4 kq = reinterpret_cast<const uint4 *>(c.data + (krow0 + r16) * kRowBytes)[g];
+    // V: dword r16 (dims 8 r16 ..) of tokens 4g .. 4g+3
+    uint32_t vd[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) vd[i] = reinterpret_cast<const uint32_t *>(c.data + (vrow0 + 4 * g + i) * kRowBytes)[r16];
+    const uint4 kpar = *reinterpret_cast<const uint4 *>(c.param + krow0 + 4 * g);
+    const uint4 vpar = *reinterpret_cast<const uint4 *>(c.param + vrow0 + 4 * g);
+
+    v4f sacc = {0.f, 0.f, 0.f, 0.f};
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.x), qop[0], sacc, 0, 0, 0);
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.y), qop[1], sacc, 0, 0, 0);
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.z), qop[2], sacc, 0, 0, 0);
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.w), qop[3], sacc, 0, 0, 0);
+
+    const uint32_t kp[4] = {kpar.x, kpar.y, kpar.z, kpar.w}, vp[4] = {vpar.x, vpar.y, vpar.z, vpar.w};
+    float sc[4], mx = m_run;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const float ks = from_bits<BF16>(kp[v]), kz = from_bits<BF16>(kp[v] >> 16);
+      sc[v] = (t0 + 4 * g + v < len) ? (ks * sacc[v] - kz * qsum) * sm_scale_log2 : kNegBig;
+      mx = fmaxf(mx, sc[v]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float corr = __builtin_amdgcn_exp2f(m_run - mx);
+    m_run = mx;
+    v4h pa;
+    float psum = 0.0f, pasum = 0.0f, pz = 0.0f;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const bool valid = t0 + 4 * g + v < len;           // rows past the end may hold anything
+      const float pv = __builtin_amdgcn_exp2f(sc[v] - mx);
+      const float vs = valid ? from_bits<BF16>(vp[v]) : 0.0f, vz = valid ? from_bits<BF16>(vp[v] >> 16) : 0.0f;
+      psum += pv;
+      pz = __builtin_fmaf(pv, vz, pz);
+      pa[v] = (_Float16)(pv * vs);
+      pasum += (float)pa[v];
+    }
+    l_run = l_run * corr + psum;
+    d_run = d_run * corr + 1024.0f * pasum;
+    z_run = z_run * corr + pz;
+    if (__any(corr != 1.0f)) {  // the running maximum of some head moved: rescale the accumulators
+      float cr[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        cr[v] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, corr), v));
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) oacc[j][v] *= cr[v];
+    }
+    // V operands: byte bb of the four token dwords -> codes 2bb (low nibbles) and 2bb+1 (high nibbles)
+#define ARCQ_PV(BB)                                                                                             \
+  {                                                                                                             \
+    const uint32_t x01 = __builtin_amdgcn_perm(vd[1], vd[0], 0x0c0c0400u + 0x00000101u * (BB));                 \
+    const uint32_t x23 = __builtin_amdgcn_perm(vd[3], vd[2], 0x0c0c0400u + 0x00000101u * (BB));                 \
+    const uint32_t t01 = __builtin_amdgcn_perm(0u, x01, 0x0c010c00u), t23 = __builtin_amdgcn_perm(0u, x23, 0x0c010c00u); \
+    v2u lo, hi;                                                                                                 \
+    lo[0] = (t01 & 0x000f000fu) | 0x64006400u;                                                                  \
+    lo[1] = (t23 & 0x000f000fu) | 0x64006400u;                                                                  \
+    hi[0] = (t01 & 0x00f000f0u) | 0x64006400u;                                                                  \
+    hi[1] = (t23 & 0x00f000f0u) | 0x64006400u;                                                                  \
+    oacc[2 * (BB)] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa, __builtin_bit_cast(v4h, lo), oacc[2 * (BB)], 0, 0, 0);      \
+    oacc[2 * (BB) + 1] =                                                                                        \
+        __builtin_amdgcn_mfma_f32_16x16x16f16(pa, __builtin_bit_cast(v4h, hi), oacc[2 * (BB) + 1], 0, 0, 0);    \
+  }
+    ARCQ_PV(0) ARCQ_PV(1) ARCQ_PV(2) ARCQ_PV(3)
+#undef ARCQ_PV
+  }
+
+  // per-wave totals of the softmax sums over the four lane groups, then merge the four waves
+  l_run += __shfl_xor(l_run, 16);
+  l_run += __shfl_xor(l_run, 32);
+  d_run += __shfl_xor(d_run, 16);
+  d_run += __shfl_xor(d_run, 32);
+  z_run += __shfl_xor(z_run, 16);
+  z_run += __shfl_xor(z_run, 32);
+  if (g == 0) {
+    if (r16 < G) {
+      part_s[wave][r16][0] = m_run;
+      part_s[wave][r16][1] = l_run;
+      part_s[wave][r16][2] = d_run;
+      part_s[wave][r16][3] = z_run;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int v = 0; v < G; ++v) part_o[wave][v][8 * r16 + j] = oacc[j][v];   // rows 4g+v = heads, g == 0
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < G * kHeadDim; idx += 256) {
+    const int hh = idx / kHeadDim, dim = idx - hh * kHeadDim;
+    float M = kNegBig;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, part_s[w][hh][0]);
+    const float unscale = (dim & 1) ? 0.0625f : 1.0f;  // odd dims were accumulated as 16 n
+    float num = 0.0f, den = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float wgt = __builtin_amdgcn_exp2f(part_s[w][hh][0] - M);
+      num = __builtin_fmaf(wgt, (part_o[w][hh][dim] - part_s[w][hh][2]) * unscale - part_s[w][hh][3], num);
+      den = __builtin_fmaf(wgt, part_s[w][hh][1], den);
+    }
+    const float out = den > 0.0f ? num / den : 0.0f;
+    o[((size_t)b * num_qo_heads + h * G + hh) * kHeadDim + dim] = (uint16_t)to_bits<BF16>(out);
+  }
+}
+
 int check_layout(const void *kv_data, const void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
                  const int32_t *last_page_offset, int n_layers, int layer_idx, int heads, int page_size, int head_dim,
                  int dtype) {
@@ -369,8 +568,15 @@ int arcq_kv_decode_i4(void *o, const void *q, int dtype, int batch, int num_qo_h
   hipStream_t st = static_cast<hipStream_t>(stream);
   uint16_t *op = static_cast<uint16_t *>(o);
   const uint16_t *qp = static_cast<const uint16_t *>(q);
-#define ARCQ_LAUNCH_DECODE(BF, GG) \
-  hipLaunchKernelGGL((kv_decode_i4_kernel<BF, GG>), grid, dim3(256), 0, st, op, qp, c, num_qo_heads, sl2)
+  static const bool force_valu = getenv("ARCQ_KV_DECODE_VALU") != nullptr;
+  const bool mfma = page_size % 16 == 0 && !force_valu;
+#define ARCQ_LAUNCH_DECODE(BF, GG)                                                                                \
+  do {                                                                                                            \
+    if (mfma)                                                                                                     \
+      hipLaunchKernelGGL((kv_decode_i4_mfma_kernel<BF, GG>), grid, dim3(256), 0, st, op, qp, c, num_qo_heads, sl2); \
+    else                                                                                                          \
+      hipLaunchKernelGGL((kv_decode_i4_kernel<BF, GG>), grid, dim3(256), 0, st, op, qp, c, num_qo_heads, sl2);    \
+  } while (0)
   if (dtype == ARCQ_DTYPE_BF16) {
     if (G == 1) ARCQ_LAUNCH_DECODE(true, 1);
     else if (G == 2) ARCQ_LAUNCH_DECODE(true, 2);

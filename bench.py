@@ -251,14 +251,18 @@ def layer_rows(torch, iters=10):
         del layer, W, kv, x, cache, cache2, step
         torch.cuda.empty_cache()
 
-    # Mixtral block, NVFP4 (benchmark configuration 5), select_num 128
+    # Mixtral block (benchmark configuration 5: NVFP4; MXFP4 beside it), select_num 128
     E, ffn, tokens = 8, 14336, 4096
     g = torch.Generator().manual_seed(5)
-    block = layers.build_mixtral_block(hidden, ffn, E, 2, 128, "NVFP4", seed=5)
     x = torch.randn(1, tokens, hidden, generator=g).to(torch.bfloat16).cuda()
     bias = torch.log(1.0 / torch.arange(1, E + 1).float() ** 1.1)
     logits = (torch.randn(tokens, E, generator=g) + bias).cuda()
-    ms_arc = timed(lambda: block(x, router_logits=logits))
+    moe_ms = {}
+    for fmt in ("NVFP4", "MXFP4"):
+        block = layers.build_mixtral_block(hidden, ffn, E, 2, 128, fmt, seed=5)
+        moe_ms[fmt] = timed(lambda: block(x, router_logits=logits))
+        del block
+        torch.cuda.empty_cache()
     # the same block in bf16 on dequantised-size weights (random: only the time matters)
     w13 = [torch.randn(2 * ffn, hidden, device="cuda", dtype=torch.bfloat16) * 0.02 for _ in range(E)]
     w2 = [torch.randn(hidden, ffn, device="cuda", dtype=torch.bfloat16) * 0.02 for _ in range(E)]
@@ -285,10 +289,11 @@ def layer_rows(torch, iters=10):
 
     ms_bf = timed(bf16_moe)
     counts = torch.bincount(torch.topk(F.softmax(logits, dim=1), 2, dim=-1)[1].reshape(-1), minlength=E).tolist()
-    rows.append({"config": "Mixtral MoE block, 4096 tokens, 8 experts top-2", "fmt": "NVFP4", "arc_ms": round(ms_arc, 3),
-                 "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_arc, 2), "tokens_per_expert": counts,
-                 "tokens_per_s": round(tokens / ms_arc * 1e3)})
-    print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
+    for fmt, ms_arc in moe_ms.items():
+        rows.append({"config": "Mixtral MoE block, 4096 tokens, 8 experts top-2", "fmt": fmt, "arc_ms": round(ms_arc, 3),
+                     "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_arc, 2), "tokens_per_expert": counts,
+                     "tokens_per_s": round(tokens / ms_arc * 1e3)})
+        print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
     return rows
 
 

@@ -100,9 +100,10 @@ def test_store_prequantized_rows(kvc, ref):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page_size", [16, 8, 32])          # 8: the VALU kernel; multiples of 16: the MFMA kernel
 @pytest.mark.parametrize("q_heads,kv_heads", [(4, 4), (8, 4), (32, 8)])
-def test_decode_attention(kvc, ref, dtype, q_heads, kv_heads):
-    batch, page_size, layers, layer = 4, 16, 2, 0
+def test_decode_attention(kvc, ref, dtype, q_heads, kv_heads, page_size):
+    batch, layers, layer = 4, 2, 0
     lengths = [1, 16, 77, 260]
     g = torch.Generator().manual_seed(5)
     total = sum(lengths)
@@ -111,11 +112,11 @@ def test_decode_attention(kvc, ref, dtype, q_heads, kv_heads):
     q = torch.randn(batch, q_heads, 128, generator=g).to(dtype)
     indptr, indices, last, maxc = make_table(lengths, page_size, batch)
     pages = torch.zeros(maxc * batch, layers, 2, kv_heads, page_size, 64, dtype=torch.uint8, device="cuda")
-    params = torch.zeros(maxc * batch, layers, 2, kv_heads, page_size, 2, dtype=dtype, device="cuda")
-    offs = [0]
+    params = torch.full((maxc * batch, layers, 2, kv_heads, page_size, 2), float("nan"), dtype=dtype, device="cuda")
+    offs = [0]                                               # unused rows hold NaN: they must not leak into results
     for n in lengths:
         offs.append(offs[-1] + n)
-    print(f"kv decode {dtype} heads {q_heads}/{kv_heads}", flush=True)
+    print(f"kv decode {dtype} heads {q_heads}/{kv_heads} page {page_size}", flush=True)
     kvc.quantize_append(pages, params, indptr.cuda(), indices.cuda(), last.cuda(), k.cuda(), v.cuda(), layer,
                         seqlen_indptr=torch.tensor(offs, dtype=torch.int32).cuda())
     o = torch.empty_like(q).cuda()
