@@ -344,7 +344,6 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
     for (int i = 0; i < WN * 2; ++i) lds_dma16(wsrc[i] + koff, lw0 + st * (BN * 128) + i * 4096);
 #pragma unroll
     for (int i = 0; i < WM * 2; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * 4096);
-#ifndef ARCQ_PROBE_NO_SCALE_DMA
     if ((kt & 1) == 0) {  // scales of steps kt and kt+1
       const int pair = kt >> 1, sst = pair & 1;
       const int soff = pair * 16 - (pair == npairs - 1 ? sc_shift : 0);
@@ -355,7 +354,6 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
       for (int j = 0; j < WM; ++j)
         if (((j + WN) & 3) == wave) lds_dma16(xssrc[j] + soff, lxs0 + sst * (BM * 16) + j * 1024);
     }
-#endif
   };
 
   // ---- LDS -> MFMA operands
@@ -434,12 +432,8 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
   issue(0);
   for (int kt = 0; kt < nfull; ++kt) {
     wait_dma_and_sync();  // stage kt&1 holds step kt; everyone is done with the other stage
-#ifndef ARCQ_PROBE_NO_DMA
     if (kt + 1 < nk) issue(kt + 1);
-#endif
-#ifndef ARCQ_PROBE_NO_COMPUTE
     compute(kt, std::false_type{});
-#endif
   }
   if (short_last) {
     wait_dma_and_sync();
@@ -919,7 +913,10 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
   if (fast_ok && (force == 1 || (force < 0 && M <= skinny_max && skinny_wins)) && M <= 64) {
     return fmt == ARCQ_FMT_MXFP4 ? launch_skinny_for<ARCQ_FMT_MXFP4>(p, st) : launch_skinny_for<ARCQ_FMT_NVFP4>(p, st);
   }
-  if (fmt == ARCQ_FMT_MXFP4 && force != 0 && fast_ok) {
+  // the tiled kernels fetch scale bytes in 16-byte windows that are shifted back at the end of a row:
+  // the row must be at least one window long (K' >= 512 for MXFP4, 256 for NVFP4)
+  const bool tiled_ok = fast_ok && Kp >= 512;
+  if (fmt == ARCQ_FMT_MXFP4 && force != 0 && tiled_ok) {
     // Tile choice from a small cost model: rounds of resident workgroups x cost of one round.
     // 256x256 tiles run ~1.3x faster per flop than 256x128 ones (LDS reads per MFMA) and 128x128
     // ones ~0.75x; 128x128 workgroups fit two to a CU.  Units: a 256x128 tile = 2.
@@ -934,7 +931,7 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
     if (force == 22 || (force < 0 && pick == 22)) return launch_mxfp4_tiled<2, 2>(p, st);
     if (force == 21 || force < 0) return launch_mxfp4_tiled<2, 1>(p, st);
   }
-  if (fmt == ARCQ_FMT_NVFP4 && force != 0 && fast_ok) {
+  if (fmt == ARCQ_FMT_NVFP4 && force != 0 && tiled_ok) {
     if (force == 44 || (force < 0 && M > 1024)) return launch_nvfp4_tiled<4, 4>(p, st);
     if (force == 42) return launch_nvfp4_tiled<4, 2>(p, st);
     if (force == 34) return launch_nvfp4_tiled<3, 4>(p, st);
