@@ -83,15 +83,18 @@ __device__ __forceinline__ float row16_max(float v) {
 // 16 lanes per row (8 values each), one wave = 4 rows.
 // ---------------------------------------------------------------------------------------------
 template <bool BF16>
-__device__ __forceinline__ void quantize_row_store(const uint16_t *src, const KvLayout &c, size_t row, int lane16) {
-  const uint4 raw = reinterpret_cast<const uint4 *>(src)[lane16];
+__device__ __forceinline__ void unpack8(const uint4 raw, float (&x)[8]) {
   const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-  float x[8];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     x[2 * i] = from_bits<BF16>(w[i]);
     x[2 * i + 1] = from_bits<BF16>(w[i] >> 16);
   }
+}
+
+// x: this lane's 8 values of the row (values of the tensor dtype)
+template <bool BF16>
+__device__ __forceinline__ void quantize_values_store(const float (&x)[8], const KvLayout &c, size_t row, int lane16) {
   float mx = x[0], mn = x[0];
 #pragma unroll
   for (int i = 1; i < 8; ++i) {
@@ -113,6 +116,70 @@ __device__ __forceinline__ void quantize_row_store(const uint16_t *src, const Kv
   }
   reinterpret_cast<uint32_t *>(c.data + row * kRowBytes)[lane16] = packed;
   if (lane16 == 0) c.param[row] = to_bits<BF16>(scale) | (to_bits<BF16>(zero) << 16);
+}
+
+template <bool BF16>
+__device__ __forceinline__ void quantize_row_store(const uint16_t *src, const KvLayout &c, size_t row, int lane16) {
+  float x[8];
+  unpack8<BF16>(reinterpret_cast<const uint4 *>(src)[lane16], x);
+  quantize_values_store<BF16>(x, c, row, lane16);
+}
+
+// ---------------------------------------------------------------------------------------------
+// decode step: rotary embedding of the new token's query and key heads and the append of its key
+// and value heads in one launch.  qkv [batch, ld]: per sequence the query heads, then the key
+// heads, then the value heads, 128 values each (the output row of a fused qkv projection).
+// Rotary embedding as torch evaluates q * cos + rotate_half(q) * sin on tensors of the model dtype
+// (model/qLlamaLayer.py:30-64, 316-321): each product and the sum rounded to that dtype, with
+// rotate_half(x) = (-x[64:], x[:64]).  cos / sin come from tables [positions, 64] in the model dtype
+// (both halves of the 128 share them).  The rotated keys and the values are quantized and stored as
+// in kv_append_i4_kernel; the rotated queries go to q_out [batch, query heads, 128].
+// 16 lanes per head row, 8 values each: the partner of value e is value e +- 64, in lane +- 8.
+// ---------------------------------------------------------------------------------------------
+template <bool BF16>
+__global__ __launch_bounds__(256) void rope_kv_append_i4_kernel(const uint16_t *qkv, int ld, const uint16_t *cos_t,
+                                                                const uint16_t *sin_t, int max_positions,
+                                                                const int32_t *positions, uint16_t *q_out,
+                                                                int num_qo_heads, KvLayout c) {
+  const int b = blockIdx.x;
+  const int lane16 = threadIdx.x & 15;
+  const int rows = num_qo_heads + 2 * c.heads;
+  const int p0 = c.indptr[b], np = c.indptr[b + 1] - p0;
+  const int len = (np - 1) * c.page_size + c.last_page_offset[b];  // length after the append
+  const int page = c.indices[p0 + (len - 1) / c.page_size], slot = (len - 1) % c.page_size;
+  const int pos = min(max(positions[b], 0), max_positions - 1);
+  for (int r = blockIdx.y * 16 + (threadIdx.x >> 4); r < rows; r += gridDim.y * 16) {
+    const uint4 raw = reinterpret_cast<const uint4 *>(qkv + (size_t)b * ld + (size_t)r * kHeadDim)[lane16];
+    float x[8];
+    unpack8<BF16>(raw, x);
+    if (r < num_qo_heads + c.heads) {  // a query or key head: rotate
+      float xp[8], cs[8], sn[8];
+      uint4 praw;
+      praw.x = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)raw.x, 0x128, 0xf, 0xf, true);  // row_ror:8 = lane ^ 8
+      praw.y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)raw.y, 0x128, 0xf, 0xf, true);
+      praw.z = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)raw.z, 0x128, 0xf, 0xf, true);
+      praw.w = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)raw.w, 0x128, 0xf, 0xf, true);
+      unpack8<BF16>(praw, xp);
+      const size_t t = (size_t)pos * (kHeadDim / 2) + 8 * (lane16 & 7);
+      unpack8<BF16>(*reinterpret_cast<const uint4 *>(cos_t + t), cs);
+      unpack8<BF16>(*reinterpret_cast<const uint4 *>(sin_t + t), sn);
+      const float sgn = lane16 < 8 ? -1.0f : 1.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = rn<BF16>(rn<BF16>(x[i] * cs[i]) + rn<BF16>((sgn * xp[i]) * sn[i]));
+    }
+    if (r < num_qo_heads) {
+      uint4 o;
+      o.x = to_bits<BF16>(x[0]) | (to_bits<BF16>(x[1]) << 16);
+      o.y = to_bits<BF16>(x[2]) | (to_bits<BF16>(x[3]) << 16);
+      o.z = to_bits<BF16>(x[4]) | (to_bits<BF16>(x[5]) << 16);
+      o.w = to_bits<BF16>(x[6]) | (to_bits<BF16>(x[7]) << 16);
+      reinterpret_cast<uint4 *>(q_out + ((size_t)b * num_qo_heads + r) * kHeadDim)[lane16] = o;
+    } else {
+      const int kv = r >= num_qo_heads + c.heads ? 1 : 0;
+      const int head = r - num_qo_heads - kv * c.heads;
+      quantize_values_store<BF16>(x, c, kv_row(c, page, kv, head, slot), lane16);
+    }
+  }
 }
 
 template <bool BF16>
@@ -512,6 +579,36 @@ int arcq_kv_append_i4(const void *k, const void *v, int dtype, int batch, const 
   else
     hipLaunchKernelGGL(kv_append_i4_kernel<false>, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint16_t *>(k), static_cast<const uint16_t *>(v), seqlen_indptr, c);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+int arcq_rope_kv_append_i4(const void *qkv, int ld, int dtype, int batch, int num_qo_heads, const void *cos_table,
+                           const void *sin_table, int max_positions, const int32_t *positions, void *q_out,
+                           void *kv_data, void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
+                           const int32_t *last_page_offset, int n_layers, int layer_idx, int num_kv_heads, int page_size,
+                           int head_dim, void *stream) {
+  using namespace arcq;
+  const int rc = check_layout(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, n_layers, layer_idx,
+                              num_kv_heads, page_size, head_dim, dtype);
+  if (rc != ARCQ_OK) return rc;
+  const long rows = (long)num_qo_heads + 2L * num_kv_heads;
+  if (batch < 0 || num_qo_heads < 1 || max_positions < 1 || ld < rows * kHeadDim || ld % 8 != 0) return ARCQ_ERR_SHAPE;
+  if (batch == 0) return ARCQ_OK;
+  if (!qkv || !cos_table || !sin_table || !positions || !q_out) return ARCQ_ERR_NULL;
+  if (!aligned16(qkv) || !aligned16(cos_table) || !aligned16(sin_table) || !aligned16(q_out)) return ARCQ_ERR_ALIGN;
+  KvLayout c{static_cast<uint8_t *>(kv_data), static_cast<uint32_t *>(kv_param), kv_indptr, kv_indices,
+             last_page_offset,               n_layers,                           layer_idx, num_kv_heads, page_size};
+  dim3 grid(batch, (unsigned)((rows + 15) / 16));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ARCQ_DTYPE_BF16)
+    hipLaunchKernelGGL(rope_kv_append_i4_kernel<true>, grid, dim3(256), 0, st, static_cast<const uint16_t *>(qkv), ld,
+                       static_cast<const uint16_t *>(cos_table), static_cast<const uint16_t *>(sin_table), max_positions,
+                       positions, static_cast<uint16_t *>(q_out), num_qo_heads, c);
+  else
+    hipLaunchKernelGGL(rope_kv_append_i4_kernel<false>, grid, dim3(256), 0, st, static_cast<const uint16_t *>(qkv), ld,
+                       static_cast<const uint16_t *>(cos_table), static_cast<const uint16_t *>(sin_table), max_positions,
+                       positions, static_cast<uint16_t *>(q_out), num_qo_heads, c);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }

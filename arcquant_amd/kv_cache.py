@@ -81,6 +81,45 @@ def quantize_append(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, 
     _lib.check(rc, "arcq_kv_append_i4")
 
 
+def rope_tables(max_positions, head_dim, dtype, device, base=10000.0):
+    """cos / sin [max_positions, head_dim/2] in `dtype`, computed as the rotary embedding of the layers
+    computes them per step (fp32 position x inverse frequency, cos / sin in fp32, cast)."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, device=device).float() / head_dim))
+    freqs = torch.outer(torch.arange(max_positions, device=device, dtype=torch.float32), inv_freq)
+    return freqs.cos().to(dtype).contiguous(), freqs.sin().to(dtype).contiguous()
+
+
+def rope_quantize_append(qkv, num_qo_heads, cos_table, sin_table, positions, kv_data, kv_param, kv_indptr, kv_indices,
+                         last_page_offset, layer_idx, q_out=None):
+    """One decode step between the qkv projection and the attention (model/qLlamaLayer.py:316-327):
+    rotary embedding of the new token's query and key heads, quantized append of its key and value heads.
+    qkv [batch, (num_qo_heads + 2 * kv_heads) * 128] (rows may be strided); returns the rotated queries
+    [batch, num_qo_heads, 128].  The page table describes the cache after the append."""
+    n_layers, heads, page_size, head_dim = _container_dims(kv_data, kv_param)
+    _check_table(kv_indptr, kv_indices, last_page_offset)
+    batch = last_page_offset.numel()
+    if qkv.dim() != 2 or qkv.shape[0] != batch or qkv.dtype != kv_param.dtype or qkv.stride(1) != 1:
+        raise RuntimeError("qkv must be [batch, (query heads + 2 * kv heads) * head_dim] in kv_param's dtype")
+    if qkv.shape[1] < (num_qo_heads + 2 * heads) * head_dim:
+        raise RuntimeError("qkv rows are too short for the head counts")
+    for t in (cos_table, sin_table):
+        if t.dtype != qkv.dtype or t.dim() != 2 or t.shape[1] != head_dim // 2 or not t.is_contiguous():
+            raise RuntimeError("cos / sin tables must be contiguous [positions, head_dim/2] of qkv's dtype")
+    if positions.dtype != torch.int32 or positions.numel() != batch or not positions.is_cuda:
+        raise RuntimeError("positions must be an int32 CUDA tensor [batch]")
+    if q_out is None:
+        q_out = torch.empty(batch, num_qo_heads, head_dim, dtype=qkv.dtype, device=qkv.device)
+    with torch.cuda.device(qkv.device):
+        rc = _lib.lib().arcq_rope_kv_append_i4(_ptr(qkv), int(qkv.stride(0)), _DTYPES[qkv.dtype], batch,
+                                               int(num_qo_heads), _ptr(cos_table), _ptr(sin_table),
+                                               int(cos_table.shape[0]), _ptr(positions), _ptr(q_out), _ptr(kv_data),
+                                               _ptr(kv_param), _ptr(kv_indptr), _ptr(kv_indices),
+                                               _ptr(last_page_offset), n_layers, int(layer_idx), heads, page_size,
+                                               head_dim, _stream(qkv))
+    _lib.check(rc, "arcq_rope_kv_append_i4")
+    return q_out
+
+
 def _store(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, seqlen_indptr, layer_idx):
     n_layers, heads, page_size, head_dim = _container_dims(kv_data, kv_param)
     _check_table(kv_indptr, kv_indices, last_page_offset)
@@ -159,6 +198,7 @@ class MultiLayerPagedKVCache4Bit:
         self._indptr, self._indices, self._last = mk(batch_size + 1), mk(max(1, max_page_cnt * batch_size)), mk(batch_size)
         self.positions = mk(batch_size)
         self._specs = None
+        self._rope = None                         # cos / sin tables of decode_step, built on first use
         self.external_step = False                # True: the caller advances the cache with begin_step()
 
     def page_cnt_from_length(self, length):
@@ -252,6 +292,22 @@ class MultiLayerPagedKVCache4Bit:
         quantize_append(k=key_states.reshape(b_sz, heads, head_dim).contiguous(),
                         v=value_states.reshape(b_sz, heads, head_dim).contiguous(), layer_idx=layer_idx, **self._specs)
         return functools.partial(self._attend, layer_idx=layer_idx)
+
+    def decode_step(self, qkv, num_qo_heads, layer_idx):
+        """The decode step of one layer from its fused qkv projection [batch, (q + 2 kv heads) * 128]:
+        rotary embedding at the positions of the new tokens, quantized append, attention over the pages.
+        Returns [batch, num_qo_heads * 128]."""
+        assert not self._needs_init[layer_idx], "decode_step comes after the prefill of this layer"
+        if layer_idx == 0 and not self.external_step:
+            self._advance_one_token()
+        if self._rope is None:
+            self._rope = rope_tables(self.pages.shape[0] // self.batch_size * self.page_size, self.head_dim,
+                                     self.scales.dtype, self.device)
+        q = rope_quantize_append(qkv, num_qo_heads, self._rope[0], self._rope[1], self.positions,
+                                 layer_idx=layer_idx, **self._specs)
+        out = torch.empty_like(q)
+        batch_decode_i4(out, q, layer_idx=layer_idx, **self._specs)
+        return out.view(q.shape[0], -1)
 
     def _attend(self, q, layer_idx):
         batch, q_len, q_heads, head_dim = q.shape

@@ -231,6 +231,11 @@ class LlamaAttention(nn.Module):
         bsz, q_len = x[3], x[4]
         d, nh, nkv = self.head_dim, self.num_heads, self.num_kv_heads
         qkv = self.qkv_proj(x)
+        if kv_cache is not None and not isinstance(kv_cache, tuple) and q_len == 1 and \
+                not kv_cache._needs_init[layer_idx]:
+            # decode over the INT4 pages: rotary embedding + quantized append in one launch, then attention
+            out = kv_cache.decode_step(qkv.view(bsz, -1), nh, layer_idx).view(bsz, 1, nh * d)
+            return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num, self.quant_type))
         q = qkv[..., :nh * d].view(bsz, q_len, nh, d).transpose(1, 2)
         k = qkv[..., nh * d:(nh + nkv) * d].view(bsz, q_len, nkv, d).transpose(1, 2)
         v = qkv[..., (nh + nkv) * d:].view(bsz, q_len, nkv, d).transpose(1, 2)

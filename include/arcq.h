@@ -163,6 +163,25 @@ int arcq_kv_append_i4(const void *k, const void *v, int dtype, int batch, const 
                       void *kv_data, void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
                       const int32_t *last_page_offset, int n_layers, int layer_idx, int num_kv_heads, int page_size,
                       int head_dim, void *stream);
+/*
+ * One decode step's work between the qkv projection and the attention, in one launch: rotary
+ * embedding of the new token's query and key heads (apply_rotary_pos_emb, model/qLlamaLayer.py:30-64,
+ * called at :316-321, evaluated as torch does on tensors of the model dtype) and the quantized
+ * append of its key and value heads (past_key_value.update, model/qLlamaLayer.py:324-327 ->
+ * model/kv_cache.py:194-276).
+ *   qkv        [batch, ld] per sequence: num_qo_heads query heads, num_kv_heads key heads,
+ *              num_kv_heads value heads, 128 values each; ld >= that, multiple of 8
+ *   cos_table, sin_table  [max_positions, 64] in `dtype`: cos / sin of position x inverse frequency,
+ *              shared by both halves of a head
+ *   positions  int32 [batch] on the device: position of each sequence's new token (clamped into the tables)
+ *   q_out      [batch, num_qo_heads, 128] rotated queries, input of arcq_kv_decode_i4
+ * The page table describes the state AFTER the append, as for arcq_kv_append_i4.
+ */
+int arcq_rope_kv_append_i4(const void *qkv, int ld, int dtype, int batch, int num_qo_heads, const void *cos_table,
+                           const void *sin_table, int max_positions, const int32_t *positions, void *q_out,
+                           void *kv_data, void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
+                           const int32_t *last_page_offset, int n_layers, int layer_idx, int num_kv_heads, int page_size,
+                           int head_dim, void *stream);
 /* the same scatter for rows the caller has quantized already -- the exact argument set of the
  * reference's init_kv_i4 (seqlen_indptr given) and append_kv_i4 (seqlen_indptr NULL):
  * k_codes / v_codes u8 [tokens, kv_heads, 64], k_param / v_param [tokens, kv_heads, 2] */

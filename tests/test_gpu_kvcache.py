@@ -163,3 +163,47 @@ def test_cache_container_flow(kvc, ref):
                     want[b, h] = torch.softmax(s, 0) @ vd[b, :, h // gsz]
             assert rel_fro(out[:, 0], want) < 5e-3
     assert cache.get_seq_length() == 33
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_quantize_append_is_bit_exact(kvc, ref, dtype):
+    """The fused decode-step launch against the same step done with torch on the CPU: rotary embedding
+    (model/qLlamaLayer.py:30-64, every op rounded to the dtype), then the quantizer restatement.
+    Rotated queries, codes and (scale, zero) pairs must be identical; rows are strided as a slice of
+    a wider projection output would be."""
+    batch, nh, nkv, page_size, layers, layer = 3, 4, 2, 16, 2, 1
+    lengths = [17, 32, 5]                                   # lengths AFTER the append: new page, page end, short
+    g = torch.Generator().manual_seed(11)
+    width = (nh + 2 * nkv) * 128
+    wide = (torch.randn(batch, width + 64, generator=g) * 1.5).to(dtype)
+    qkv = wide[:, :width]
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32)
+    positions[2] = 40                                       # a position that differs from the length (padded prompt)
+    cos_t, sin_t = kvc.rope_tables(64, 128, dtype, "cuda")
+    indptr, indices, last, maxc = make_table(lengths, page_size, batch)
+    pages = torch.zeros(maxc * batch, layers, 2, nkv, page_size, 64, dtype=torch.uint8, device="cuda")
+    params = torch.zeros(maxc * batch, layers, 2, nkv, page_size, 2, dtype=dtype, device="cuda")
+    print(f"rope + kv append {dtype}", flush=True)
+    q_rot = kvc.rope_quantize_append(wide.cuda()[:, :width], nh, cos_t, sin_t, positions.cuda(), pages, params,
+                                     indptr.cuda(), indices.cuda(), last.cuda(), layer)
+    torch.cuda.synchronize()
+
+    # the same on the CPU, op by op
+    q = qkv[:, :nh * 128].view(batch, nh, 128)
+    k = qkv[:, nh * 128:(nh + nkv) * 128].view(batch, nkv, 128)
+    v = qkv[:, (nh + nkv) * 128:].view(batch, nkv, 128)
+    cos = torch.cat([cos_t.cpu(), cos_t.cpu()], dim=-1)[positions.long()][:, None]     # [batch, 1, 128]
+    sin = torch.cat([sin_t.cpu(), sin_t.cpu()], dim=-1)[positions.long()][:, None]
+    rot = lambda x: torch.cat((-x[..., 64:], x[..., :64]), dim=-1)
+    q_want = q * cos + rot(q) * sin
+    k_rot = k * cos + rot(k) * sin
+    assert torch.equal(q_rot.cpu(), q_want)
+    pc, sc = pages.cpu(), params.cpu()
+    assert int(pc[:, 0].sum()) == 0
+    for b in range(batch):
+        (kc, kp), (vc, vp) = ref.gather_sequence(pc, sc, indptr, indices, last, layer, b)
+        for codes, par, x in ((kc, kp, k_rot[b:b + 1]), (vc, vp, v[b:b + 1])):
+            qq, s, z = ref.asym_quantize_and_pack_i4(x)
+            assert torch.equal(codes[-1:], ref.unpack(qq))
+            assert torch.equal(par[-1:, :, 0], s[..., 0].double()) and torch.equal(par[-1:, :, 1], z[..., 0].double())
+            assert int(codes[:-1].sum()) == 0                # earlier slots untouched
