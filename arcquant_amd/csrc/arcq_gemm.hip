@@ -12,6 +12,8 @@
 #include <hip/hip_runtime.h>
 #include <stdlib.h>
 
+#include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "arcq_internal.h"
@@ -32,6 +34,10 @@ struct GemmParams {
   const float *d_alpha_a, *d_alpha_b;
   float alpha;
   int M, N, Kp;
+  // split-K (tiled kernels): blockIdx.y selects one of k_slices ranges of K steps and the workgroup
+  // writes its fp32 partial tile to partial[slice][M][N] instead of C; splitk_reduce_kernel adds them
+  float *partial = nullptr;
+  int k_slices = 1;
 };
 
 __device__ __forceinline__ float effective_alpha(const GemmParams &p) {
@@ -238,6 +244,30 @@ __device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (
   constexpr int BN = 64 * WN, BM = 64 * WM;
   const int r = lane & 31, kh = lane >> 5;
   const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;
+  if (p.partial) {  // split-K: the unscaled fp32 tile of this K range
+    float *part = p.partial + (size_t)blockIdx.y * p.M * p.N;
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
+#pragma unroll
+      for (int j = 0; j < WM; ++j) {
+        const int m = m_base + wm0 + 32 * j + r;
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n_base + wn0 + 32 * i + 8 * q + 4 * kh;
+          float *dst = part + (size_t)m * p.N + n;
+          if (n + 3 < p.N && (p.N & 3) == 0) {
+            *reinterpret_cast<float4 *>(dst) =
+                make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < p.N) dst[e] = acc[i][j][4 * q + e];
+          }
+        }
+      }
+    return;
+  }
   const float alpha = effective_alpha(p);
   constexpr bool kPow2 = (WN & (WN - 1)) == 0;  // the swizzled transpose below needs 4*WN lanes per row to be a power of two
   if (kPow2 && m_base + BM <= p.M && n_base + BN <= p.N && (p.N & 7) == 0) {
@@ -428,14 +458,19 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
 #undef ARCQ_MX_SUBSTEP
   };
 
-  const int nfull = short_last ? nk - 1 : nk;
-  issue(0);
-  for (int kt = 0; kt < nfull; ++kt) {
+  // this workgroup's K steps: all of them, or with split-K a range that starts on a pair of steps
+  // (the scale bytes travel in pairs)
+  const int kt_beg = 2 * (int)((long)npairs * blockIdx.y / p.k_slices);
+  const int kt_end = min(nk, 2 * (int)((long)npairs * (blockIdx.y + 1) / p.k_slices));
+  const bool tail = short_last && kt_end == nk;
+  const int nfull = tail ? kt_end - 1 : kt_end;
+  if (kt_beg < kt_end) issue(kt_beg);
+  for (int kt = kt_beg; kt < nfull; ++kt) {
     wait_dma_and_sync();  // stage kt&1 holds step kt; everyone is done with the other stage
-    if (kt + 1 < nk) issue(kt + 1);
+    if (kt + 1 < kt_end) issue(kt + 1);
     compute(kt, std::false_type{});
   }
-  if (short_last) {
+  if (tail && kt_beg < kt_end) {
     wait_dma_and_sync();
     compute(nk - 1, std::true_type{});
   }
@@ -650,14 +685,16 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  const int nfull = short_last ? nk - 1 : nk;
-  issue(0);
-  for (int kt = 0; kt < nfull; ++kt) {
+  const int kt_beg = (int)((long)nk * blockIdx.y / p.k_slices), kt_end = (int)((long)nk * (blockIdx.y + 1) / p.k_slices);
+  const bool tail = short_last && kt_end == nk;
+  const int nfull = tail ? kt_end - 1 : kt_end;
+  if (kt_beg < kt_end) issue(kt_beg);
+  for (int kt = kt_beg; kt < nfull; ++kt) {
     wait_dma_and_sync();
-    if (kt + 1 < nk) issue(kt + 1);
+    if (kt + 1 < kt_end) issue(kt + 1);
     compute(kt, std::false_type{});
   }
-  if (short_last) {
+  if (tail && kt_beg < kt_end) {
     wait_dma_and_sync();
     compute(nk - 1, std::true_type{});
   }
@@ -858,7 +895,7 @@ int launch_nvfp4_tiled(const GemmParams &p, hipStream_t st) {
   constexpr int BN = 64 * WN, BM = 64 * WM;
   const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   const int grid = ((total + 7) / 8) * 8;
-  hipLaunchKernelGGL((gemm_nvfp4_tiled<WN, WM>), dim3(grid), dim3(256), 0, st, p);
+  hipLaunchKernelGGL((gemm_nvfp4_tiled<WN, WM>), dim3(grid, p.k_slices), dim3(256), 0, st, p);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }
@@ -868,7 +905,63 @@ int launch_mxfp4_tiled(const GemmParams &p, hipStream_t st) {
   constexpr int BN = 64 * WN, BM = 64 * WM;
   const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   const int grid = ((total + 7) / 8) * 8;  // whole groups of 8 so that the XCD split covers every tile
-  hipLaunchKernelGGL((gemm_mxfp4_tiled<WN, WM>), dim3(grid), dim3(256), 0, st, p);
+  hipLaunchKernelGGL((gemm_mxfp4_tiled<WN, WM>), dim3(grid, p.k_slices), dim3(256), 0, st, p);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+// Split-K for few rows of activations and narrow layers: a 128x64 tile grid alone leaves most CUs idle
+// (N = 4096, M = 64: 32 workgroups), so K is cut into slices, one workgroup per (tile, slice), each
+// writing its fp32 partial tile; this kernel adds the slices in order and writes bf16.  The kernel
+// boundary makes the partials visible; nothing is accumulated atomically, so results are
+// reproducible.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p) {
+  const size_t total4 = ((size_t)p.M * p.N) >> 2, plane = (size_t)p.M * p.N;
+  const float alpha = effective_alpha(p);
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total4; i += (size_t)gridDim.x * 256) {
+    float4 t = reinterpret_cast<const float4 *>(p.partial)[i];
+    for (int k = 1; k < p.k_slices; ++k) {
+      const float4 u = reinterpret_cast<const float4 *>(p.partial + (size_t)k * plane)[i];
+      t.x += u.x, t.y += u.y, t.z += u.z, t.w += u.w;
+    }
+    const uint32_t lo = f32_to_bf16_bits(t.x * alpha) | (f32_to_bf16_bits(t.y * alpha) << 16);
+    const uint32_t hi = f32_to_bf16_bits(t.z * alpha) | (f32_to_bf16_bits(t.w * alpha) << 16);
+    reinterpret_cast<uint2 *>(p.c)[i] = make_uint2(lo, hi);
+  }
+}
+
+// Workspace of the partial tiles: one per device, allocated on the first call that needs it and kept
+// until the process ends (a captured graph may hold its address).  Calls that overlap in time on one
+// device would share it; launches are stream-ordered as everywhere else in this library.
+constexpr size_t kSplitWorkspaceBytes = 32u << 20;
+constexpr int kSplitMaxDevices = 16;
+
+inline float *splitk_workspace() {
+  static std::mutex mu;
+  static float *ws[kSplitMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSplitMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ws[dev]) {
+    float *w = nullptr;
+    if (hipMalloc(&w, kSplitWorkspaceBytes) != hipSuccess) {
+      (void)hipGetLastError();  // e.g. under stream capture before any eager call: the caller runs without split-K
+      return nullptr;
+    }
+    ws[dev] = w;
+  }
+  return ws[dev];
+}
+
+template <int FMT>
+int launch_tiled_splitk(GemmParams p, int slices, hipStream_t st) {
+  p.k_slices = slices;
+  p.partial = splitk_workspace();
+  if (!p.partial || (size_t)slices * p.M * p.N * sizeof(float) > kSplitWorkspaceBytes) return -1;
+  const int rc = FMT == ARCQ_FMT_MXFP4 ? launch_mxfp4_tiled<2, 1>(p, st) : launch_nvfp4_tiled<2, 1>(p, st);
+  if (rc != ARCQ_OK) return rc;
+  const size_t total4 = ((size_t)p.M * p.N) >> 2;
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<size_t>((total4 + 255) / 256, 1024)), dim3(256), 0, st, p);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }
@@ -910,6 +1003,23 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
   const bool skinny_wins = fmt == ARCQ_FMT_MXFP4
                                ? (N <= 4096 || (N <= 8192 && (M <= 32 || Kp >= 8192)) || M <= 4)
                                : (N <= 8192 || M <= 16);
+  // Narrow layers with a decode batch of tens of rows: 128x64 tiles with K cut into slices (measured
+  // against the skinny and the plain tiled kernels with the weights streaming from HBM; two launches,
+  // so it pays only where the single launch is far from the weight stream's time).
+  // ARCQ_GEMM_SPLITK=<slices> forces it for M <= 64, =1 switches it off.
+  static const int split_env = getenv("ARCQ_GEMM_SPLITK") ? atoi(getenv("ARCQ_GEMM_SPLITK")) : 0;
+  int split = 0;
+  if (split_env > 1) split = M <= 64 ? split_env : 0;
+  else if (split_env == 0 && force < 0 && N <= 8192) {
+    if (Kp >= 8192 && M >= 24 && M <= 64) split = 8;
+    else if (Kp < 8192 && N > 4096 && M > 32 && M <= 64) split = 4;
+  }
+  if (split > 1 && fast_ok && Kp >= 512 && (N & 3) == 0) {
+    const int slices = std::min(split, (Kp + 255) / 256 / 2);
+    const int rc = fmt == ARCQ_FMT_MXFP4 ? launch_tiled_splitk<ARCQ_FMT_MXFP4>(p, slices, st)
+                                         : launch_tiled_splitk<ARCQ_FMT_NVFP4>(p, slices, st);
+    if (rc >= 0) return rc;
+  }
   if (fast_ok && (force == 1 || (force < 0 && M <= skinny_max && skinny_wins)) && M <= 64) {
     return fmt == ARCQ_FMT_MXFP4 ? launch_skinny_for<ARCQ_FMT_MXFP4>(p, st) : launch_skinny_for<ARCQ_FMT_NVFP4>(p, st);
   }

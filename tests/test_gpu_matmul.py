@@ -113,18 +113,21 @@ def test_matmul_llama_shapes_vs_torch_fp32(agemm, fmt, M, N, K, S):
 
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 32, 48, 64])
-@pytest.mark.parametrize("N,K,S", [(6144, 4096, 256), (202, 384, 0), (4100, 1024, 128)])
+@pytest.mark.parametrize("N,K,S", [(6144, 4096, 256), (202, 384, 0), (4100, 1024, 128), (4100, 8192, 128)])
 def test_matmul_decode_batches(agemm, fmt, M, N, K, S):
     """M <= 64 (decode batches) at a benchmark shape and at shapes whose N is not a multiple of the
     16-row strips or of the 4-wide stores: against torch's fp32 matmul of the dequantized operands,
     and, row by row, against the same call on a 128-row batch that contains these rows (another
-    kernel computes that one)."""
+    kernel computes that one).  The long-K shape and the wider batches of the benchmark shape take the
+    split-K path (partial tiles in a workspace, added by a second launch): a repeated call must give
+    the same bits."""
     (x, w, idx, gx, gw), (a, sfa, b, sfb) = quantized_pair(agemm, 128, N, K, S, fmt, seed=11)
     print(f"matmul decode {fmt} M={M} N={N} K={K} S={S}", flush=True)
     a_m = a[:M].contiguous()
     sfa_m = sfa.view(128, -1)[:M].contiguous().view(-1)
     y = agemm.matmul(a_m, b, sfa_m, sfb, gx * gw)
     assert y.shape == (M, N)
+    assert torch.equal(y, agemm.matmul(a_m, b, sfa_m, sfb, gx * gw))
     prev = torch.backends.cuda.matmul.allow_tf32
     torch.backends.cuda.matmul.allow_tf32 = False
     try:
