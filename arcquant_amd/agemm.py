@@ -124,6 +124,23 @@ def rmsnorm_quantize_x(X, W, eps, reorder_index, KE, *, fmt="NVFP4", global_scal
     return _quantize("arcq_rmsnorm_quantize_x", X, W, eps, reorder_index, KE, fmt, global_scale)
 
 
+def tensor_scale(x, divisor=2688.0):
+    """NVFP4 tensor scale max|x| / divisor of bf16 activations [M, K] (rows may be strided) as a 0-dim
+    fp32 tensor on x's device, 1 for an all-zero tensor: what the reference's callers compute with torch
+    ahead of the quantizer (model/qLlamaLayer.py:73-77), in one launch."""
+    if not isinstance(x, torch.Tensor) or x.dtype != torch.bfloat16 or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
+        raise RuntimeError("tensor_scale takes a 2-D bf16 CUDA tensor with unit stride along its last dimension")
+    M, K = x.shape
+    ld = x.stride(0) if M > 1 else K
+    if K % 8 or ld % 8 or x.data_ptr() % 16:
+        raise RuntimeError(f"Value error in tensor_scale: K={K}, row stride {ld} not supported")
+    out = torch.empty((), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().arcq_tensor_scale(x.data_ptr(), None, ld, M, K, float(divisor), out.data_ptr(), _stream(x))
+    _lib.check(rc, "arcq_tensor_scale")
+    return out
+
+
 def swiglu_quantize_x(gate, up, reorder_index, KE, *, fmt="NVFP4", global_scale=None):
     """act_fn(gate) * up -> quantized activations in one pass (no counterpart in the reference's
     module; its layers do silu, multiply and quantize as separate ops, model/qLlamaLayer.py:432-439).
@@ -152,11 +169,9 @@ def swiglu_quantize_x(gate, up, reorder_index, KE, *, fmt="NVFP4", global_scale=
         if want_scale:
             if global_scale != "absmax":
                 raise RuntimeError("global_scale must be a number, a tensor or 'absmax'")
-            amax = torch.zeros((), dtype=torch.float32, device=gate.device)
-            _lib.check(L.arcq_swiglu_absmax(gate.data_ptr(), up.data_ptr(), ld, M, K, amax.data_ptr(), _stream(gate)),
-                       "arcq_swiglu_absmax")
-            global_scale = amax / torch.full_like(amax, 2688.0)
-            global_scale = torch.where(global_scale == 0, torch.ones_like(global_scale), global_scale)
+            global_scale = torch.empty((), dtype=torch.float32, device=gate.device)
+            _lib.check(L.arcq_tensor_scale(gate.data_ptr(), up.data_ptr(), ld, M, K, 2688.0, global_scale.data_ptr(),
+                                           _stream(gate)), "arcq_tensor_scale")
         gs, d_gs, keep = _scalar(global_scale, gate.device)
         QX = torch.empty((M, (K + KE) // 2), dtype=torch.uint8, device=gate.device)
         SFX = torch.empty((L.arcq_scales_bytes(M, K, KE, f),), dtype=torch.uint8, device=gate.device)

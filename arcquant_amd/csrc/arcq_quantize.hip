@@ -9,6 +9,8 @@
 #include <hip/hip_runtime.h>
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "arcq_internal.h"
 #include "arcq_math.h"
 
@@ -604,6 +606,76 @@ __global__ __launch_bounds__(256) void swiglu_absmax_kernel(const uint16_t *gate
   if ((threadIdx.x & 63) == 0 && m) atomicMax(out, m);
 }
 
+// NVFP4 tensor scale of an activation tensor in one launch: max |x| / divisor (model/qLlamaLayer.py:74),
+// 1 for an all-zero tensor, as an fp32 scalar on the device.  SWIGLU: x = act_fn(gate) * up formed on the
+// fly.  Blocks meet through two words of a persistent workspace (running maximum as the bits of a
+// non-negative float, arrival counter): the last block to arrive divides, writes the scale and puts
+// both words back to zero.  Only device-scope atomics touch the two words, and a block's arrival is
+// issued after its maximum has returned, so the last block reads the maximum of all of them.
+template <bool SWIGLU>
+__global__ __launch_bounds__(256) void tensor_scale_kernel(const uint16_t *x, const uint16_t *up, size_t ld, int rows,
+                                                           int K, float divisor, uint32_t *ws, float *out) {
+  __shared__ uint32_t wave_max[4];
+  const int cpr = K >> 3;  // 16-byte chunks per row
+  const size_t total = (size_t)rows * cpr;
+  uint32_t m = 0u;
+  for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < total; c += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = c / cpr, k = (c % cpr) << 3;
+    const uint4 g = *reinterpret_cast<const uint4 *>(x + r * ld + k);
+    uint32_t t[4] = {g.x, g.y, g.z, g.w};
+    if (SWIGLU) {
+      const uint4 u = *reinterpret_cast<const uint4 *>(up + r * ld + k);
+      t[0] = swiglu_pair(g.x, u.x), t[1] = swiglu_pair(g.y, u.y), t[2] = swiglu_pair(g.z, u.z), t[3] = swiglu_pair(g.w, u.w);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t lo = (t[i] << 16) & 0x7fffffffu, hi = t[i] & 0x7fff0000u;
+      m = lo > m ? lo : m;
+      m = hi > m ? hi : m;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint32_t v = (uint32_t)__shfl_xor((int)m, o);
+    m = v > m ? v : m;
+  }
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  for (int w = 1; w < 4; ++w) m = wave_max[w] > m ? wave_max[w] : m;
+  const uint32_t old = atomicMax(ws, m);                        // old < 2^31: the next line waits for it
+  const uint32_t arrived = atomicAdd(ws + 1, 1u + (old >> 31));
+  if (arrived != gridDim.x - 1) return;
+  const float amax = u2f(atomicMax(ws, 0u));
+  const float scale = amax / divisor;
+  *out = scale == 0.0f ? 1.0f : scale;
+  atomicExch(ws, 0u);
+  atomicExch(ws + 1, 0u);
+}
+
+// the two workspace words, one pair per device, allocated (and zeroed) on first use and kept
+inline uint32_t *tensor_scale_workspace() {
+  static std::mutex mu;
+  static uint32_t *ws[16];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ws[dev]) {
+    uint32_t *w = nullptr;
+    if (hipMalloc(&w, 2 * sizeof(uint32_t)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    if (hipMemset(w, 0, 2 * sizeof(uint32_t)) != hipSuccess) {
+      (void)hipGetLastError();
+      (void)hipFree(w);
+      return nullptr;
+    }
+    ws[dev] = w;
+  }
+  return ws[dev];
+}
+
 template <int FMT, int MODE, bool SCALED>
 int launch_quantize_unit(const QuantParams &p, hipStream_t stream) {
   const int threads = (((p.K >> 4) + 63) / 64) * 64;
@@ -844,6 +916,26 @@ int arcq_swiglu_absmax(const void *gate, const void *up, int ld, int M, int K, f
   hipLaunchKernelGGL(arcq::swiglu_absmax_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const uint16_t *>(gate), static_cast<const uint16_t *>(up), (size_t)ld, M, K,
                      reinterpret_cast<uint32_t *>(d_absmax));
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+int arcq_tensor_scale(const void *x, const void *up, int ld, int M, int K, float divisor, float *d_scale, void *stream) {
+  if (M < 0 || K < 8 || K % 8 != 0 || ld < K || ld % 8 != 0 || !(divisor > 0.0f)) return ARCQ_ERR_SHAPE;
+  if (!x || !d_scale) return ARCQ_ERR_NULL;
+  if (!arcq::aligned16(x) || (up && !arcq::aligned16(up))) return ARCQ_ERR_ALIGN;
+  uint32_t *ws = arcq::tensor_scale_workspace();
+  if (!ws) return ARCQ_ERR_LAUNCH;
+  const size_t chunks = (size_t)M * (K >> 3);
+  int grid = (int)((chunks + 255) / 256 < 1024 ? (chunks + 255) / 256 : 1024);
+  if (grid < 1) grid = 1;  // M == 0: one block writes the scale of an empty tensor, 1
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (up)
+    hipLaunchKernelGGL(arcq::tensor_scale_kernel<true>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(x),
+                       static_cast<const uint16_t *>(up), (size_t)ld, M, K, divisor, ws, d_scale);
+  else
+    hipLaunchKernelGGL(arcq::tensor_scale_kernel<false>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(x),
+                       static_cast<const uint16_t *>(nullptr), (size_t)ld, M, K, divisor, ws, d_scale);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }

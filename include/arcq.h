@@ -120,6 +120,19 @@ int arcq_swiglu_quantize_x(const void *gate, const void *up, int ld, int M, int 
 int arcq_swiglu_absmax(const void *gate, const void *up, int ld, int M, int K, float *d_absmax, void *stream);
 
 /*
+ * NVFP4 tensor scale of an activation tensor, max |x| / divisor, as the reference's callers compute it
+ * with torch before the quantizer (x.abs().max() / (448 * 6), model/qLlamaLayer.py:73-77), in one
+ * launch and without a host round trip; an all-zero tensor gets 1.
+ *   x        bf16 rows of K elements, row stride ld (elements, multiple of 8); K multiple of 8
+ *   up       NULL, or the second operand of a fused SwiGLU: the scale is then that of
+ *            act_fn(x) * up (x = gate), as arcq_swiglu_quantize_x forms it
+ *   d_scale  fp32 scalar on the device, read by the quantizer (d_global_scale) and the GEMM (d_alpha_a)
+ * Blocks combine their maxima through two words of a per-device workspace that the library allocates
+ * on first use and keeps; calls that overlap in time on one device would share it.
+ */
+int arcq_tensor_scale(const void *x, const void *up, int ld, int M, int K, float divisor, float *d_scale, void *stream);
+
+/*
  * Augmented-K block-scaled FP4 GEMM: C[M,N] = alpha * dq(A)[M,K'] @ dq(B)[N,K']^T, fp32
  * accumulation, bf16 output.
  * Replaces agemm.matmul (kernels/src/bindings.cpp:99-120 -> nvfp4.cu:35-132).

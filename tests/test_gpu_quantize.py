@@ -186,3 +186,24 @@ def test_errors(agemm):
     agemm.check_index(idx)
     q, sf = agemm.reorder_quantize_x(x[:0], idx, 64)               # empty input
     assert q.shape == (0, (4096 + 64) // 2) and sf.numel() == 0
+
+
+@pytest.mark.parametrize("M,K", [(1, 64), (5, 4096), (64, 14336), (2048, 4096), (300, 1000)])
+def test_tensor_scale_matches_torch(agemm, M, K):
+    """NVFP4 tensor scale in one launch (max|x| / 2688, model/qLlamaLayer.py:73-77) against torch's
+    abs().max() and an IEEE division; repeated calls reuse the library's two-word workspace, which must
+    come back clean; an all-zero tensor gets 1; strided rows are read in place."""
+    g = torch.Generator().manual_seed(100 + M)
+    x = (torch.randn(M, K + 8, generator=g) * 3).to(torch.bfloat16)
+    x[M // 2, K // 3] = -777.0                                   # the maximum is a negative element
+    x[:, K:] = 1e4                                               # outside the view: must not be read
+    xd = x.cuda()
+    view = xd[:, :K]
+    want = view.abs().max().float() / torch.full((), 2688.0, device="cuda")
+    print(f"tensor scale M={M} K={K}", flush=True)
+    for _ in range(3):
+        got = agemm.tensor_scale(view)
+        assert got.dtype == torch.float32 and got.dim() == 0
+        assert float(got) == float(want)
+    assert float(agemm.tensor_scale(torch.zeros(M, K, dtype=torch.bfloat16, device="cuda"))) == 1.0
+    assert float(agemm.tensor_scale(view.contiguous(), 6.0)) == float(view.abs().max().float() / torch.full((), 6.0, device="cuda"))
