@@ -381,7 +381,7 @@ def build_mixtral_block(hidden=4096, ffn=14336, num_experts=8, top_k=2, select_n
 
 class GraphedDecodeStep:
     """One decoder layer's decode step (one new token per sequence, INT4 paged KV cache) captured
-    once as a HIP graph and replayed: the step is a chain of ~60 short launches whose issue cost on
+    once as a HIP graph and replayed: the step is a chain of ~20 short launches whose issue cost on
     the host exceeds their run time.  Host-side cache bookkeeping happens in cache.begin_step() before
     each replay; the token positions for the rotary embedding are read from cache.positions on the
     device.  No memset nodes are recorded (buffers are cleared by fill kernels)."""

@@ -425,8 +425,10 @@ def main():
     }
 
     if not args.no_gemm:
-        shapes = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)] if args.gemm_table else [(6144, 4096)]
-        Ms = [1, 16, 64, 128, 512, 2048, 4096] if args.gemm_table else [1, 16, 512, 4096]
+        # default: the qkv and gate_up projections of Llama-3-8B (the smallest and the largest weight of a layer)
+        shapes = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)] if args.gemm_table else \
+            [(6144, 4096), (28672, 4096)]
+        Ms = [1, 16, 64, 128, 512, 2048, 4096] if args.gemm_table else [1, 16, 64, 512, 4096]
         out["gemm"] = gemm_rows(torch, agemm, shapes, Ms, ["MXFP4", "NVFP4"])
         out["gemm_peaks_tflops"] = MFMA_PEAK_TFLOPS
     if args.layers:
