@@ -310,7 +310,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; every GPU box of this run has one and nothing here shards "
-              "across devices (rows are independent, see DESIGN.md). Use --gpus 1.", file=sys.stderr)
+              "across devices (rows of every quantizer and GEMM are independent: shard M, no exchange). "
+              "Use --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import ctypes
