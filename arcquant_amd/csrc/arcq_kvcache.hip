@@ -146,7 +146,8 @@ __global__ __launch_bounds__(256) void rope_kv_append_i4_kernel(const uint16_t *
   const int rows = num_qo_heads + 2 * c.heads;
   const int p0 = c.indptr[b], np = c.indptr[b + 1] - p0;
   const int len = (np - 1) * c.page_size + c.last_page_offset[b];  // length after the append
-  const int page = c.indices[p0 + (len - 1) / c.page_size], slot = (len - 1) % c.page_size;
+  const bool has_slot = np > 0 && len > 0;                          // a table without room for the new token: no append
+  const int page = has_slot ? c.indices[p0 + (len - 1) / c.page_size] : 0, slot = has_slot ? (len - 1) % c.page_size : 0;
   const int pos = min(max(positions[b], 0), max_positions - 1);
   for (int r = blockIdx.y * 16 + (threadIdx.x >> 4); r < rows; r += gridDim.y * 16) {
     const uint4 raw = reinterpret_cast<const uint4 *>(qkv + (size_t)b * ld + (size_t)r * kHeadDim)[lane16];
@@ -174,7 +175,7 @@ __global__ __launch_bounds__(256) void rope_kv_append_i4_kernel(const uint16_t *
       o.z = to_bits<BF16>(x[4]) | (to_bits<BF16>(x[5]) << 16);
       o.w = to_bits<BF16>(x[6]) | (to_bits<BF16>(x[7]) << 16);
       reinterpret_cast<uint4 *>(q_out + ((size_t)b * num_qo_heads + r) * kHeadDim)[lane16] = o;
-    } else {
+    } else if (has_slot) {
       const int kv = r >= num_qo_heads + c.heads ? 1 : 0;
       const int head = r - num_qo_heads - kv * c.heads;
       quantize_values_store<BF16>(x, c, kv_row(c, page, kv, head, slot), lane16);

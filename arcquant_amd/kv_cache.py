@@ -195,8 +195,9 @@ class MultiLayerPagedKVCache4Bit:
         # graph of a decode step keeps reading the right addresses.  `positions` holds the position of
         # each sequence's newest token (for rotary embeddings inside a graph).
         mk = lambda n: torch.zeros(n, dtype=torch.int32, device=device)
-        self._indptr, self._indices, self._last = mk(batch_size + 1), mk(max(1, max_page_cnt * batch_size)), mk(batch_size)
-        self.positions = mk(batch_size)
+        self._indptr, self._indices = mk(batch_size + 1), mk(max(1, max_page_cnt * batch_size))
+        self._counters = mk(2 * batch_size)       # last_page_offset | positions: one add advances both
+        self._last, self.positions = self._counters[:batch_size], self._counters[batch_size:]
         self._specs = None
         self._rope = None                         # cos / sin tables of decode_step, built on first use
         self.external_step = False                # True: the caller advances the cache with begin_step()
@@ -248,8 +249,7 @@ class MultiLayerPagedKVCache4Bit:
         if new_page or self._specs is None:
             self._build_specs()
         else:
-            self._last.add_(1)
-            self.positions.add_(1)
+            self._counters.add_(1)
 
     def begin_step(self):
         """Advance every sequence by one token ahead of a decode step whose launches are replayed from

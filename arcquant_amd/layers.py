@@ -415,6 +415,7 @@ class GraphedDecodeStep:
     @torch.no_grad()
     def __call__(self, hidden_states):
         self.cache.begin_step()
-        self.x.copy_(hidden_states)
+        if hidden_states.data_ptr() != self.x.data_ptr():    # a caller may write into self.x directly
+            self.x.copy_(hidden_states)
         self.graph.replay()
         return self.y
