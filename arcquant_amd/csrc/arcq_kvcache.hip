@@ -350,9 +350,10 @@ __global__ __launch_bounds__(256) void kv_decode_i4_kernel(uint16_t *o, const ui
 // Kn, Vn are the stored codes 0..15 as fp16; scale and zero of the rows enter through the identities
 // above (s * dot - z * sum(q), and p * s_v folded into P), so no element is dequantized.
 // Codes become fp16 by or-ing them into the mantissa of 1024 (0x6400 | n = 1024 + n; the high nibble
-// of a byte lands four bits up and reads 1024 + 16 n): for K the 1024 is subtracted exactly with a
-// packed add and the factor 16 is divided out of the matching q elements; for V both are removed
-// from the accumulated sums at the end (sum_t p_t * 1024 is tracked beside the softmax denominator).
+// of a byte lands four bits up and reads 1024 + 16 n): for K the factor 16 is divided out of the
+// matching q elements and the 1024 terms leave the scores as one number per head; for V both are
+// removed from the accumulated sums at the end (sum_t p_t * 1024 is tracked beside the softmax
+// denominator).
 // Layouts make every operand a plain load: the K operand row of a lane is its token's 16 bytes
 // (the MFMA's K index is a permutation of the dims, applied to Q^T as well), S^T comes out with a
 // lane holding 4 tokens of one head, which is exactly the A operand of the second product, and the
@@ -365,32 +366,32 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
-// byte I of x into the low byte of both halves of a dword
-template <int I>
-__device__ __forceinline__ uint32_t spread_byte(uint32_t x) {
-  return __builtin_amdgcn_perm(0u, x, 0x0c000c00u | ((uint32_t)I << 16) | (uint32_t)I);
-}
-// (lo nibble, hi nibble * 16) of the spread byte as fp16, 1024 removed
-__device__ __forceinline__ uint32_t nibbles_exact(uint32_t t) {
-  typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-  const v2h v = __builtin_bit_cast(v2h, (t & 0x00f0000fu) | 0x64006400u);
-  const v2h off = {(_Float16)1024.0f, (_Float16)1024.0f};
-  return __builtin_bit_cast(uint32_t, v - off);
-}
-__device__ __forceinline__ v8h k_operand(uint32_t x) {  // 8 codes -> (n0, 16 n1, n2, 16 n3, ...)
+// 8 codes of a dword -> 8 fp16 values with the 1024 left in: bytes b0..b3 hold dims (0,1) (2,3) (4,5) (6,7) as
+// (low, high) nibbles; the result is (1024 + n0, 1024 + n4, 1024 + 16 n1, 1024 + 16 n5, 1024 + n2, 1024 + n6,
+// 1024 + 16 n3, 1024 + 16 n7): five instructions.  Q^T is laid out in the same order with the
+// elements that meet a 16 n divided by 16, and the 1024 terms are subtracted from the scores as one
+// number per head (1024 * sum of q over the low-nibble dims + 64 * sum over the high-nibble dims).
+constexpr int kDimOfElem[8] = {0, 4, 1, 5, 2, 6, 3, 7};
+__device__ __forceinline__ v8h k_operand(uint32_t x) {
   v4u d;
-  d[0] = nibbles_exact(spread_byte<0>(x));
-  d[1] = nibbles_exact(spread_byte<1>(x));
-  d[2] = nibbles_exact(spread_byte<2>(x));
-  d[3] = nibbles_exact(spread_byte<3>(x));
+  const uint32_t y = x >> 8;
+  d[0] = (x & 0x000f000fu) | 0x64006400u;
+  d[1] = (x & 0x00f000f0u) | 0x64006400u;
+  d[2] = (y & 0x000f000fu) | 0x64006400u;
+  d[3] = (y & 0x00f000f0u) | 0x64006400u;
   return __builtin_bit_cast(v8h, d);
 }
 
+// kDecodeWaves waves per workgroup share the chunks of one (sequence, KV head): a chunk is a chain of
+// dependent steps (loads, four MFMAs on one accumulator, cross-lane maxima, exponentials, eight more
+// MFMAs), so the kernel lives on waves per SIMD, and batch x KV heads workgroups of four waves give
+// only two.
+constexpr int kDecodeWaves = 8;
 template <bool BF16, int G>
-__global__ __launch_bounds__(256) void kv_decode_i4_mfma_kernel(uint16_t *o, const uint16_t *q, KvLayout c,
-                                                                int num_qo_heads, float sm_scale_log2) {
-  __shared__ float part_o[4][G][kHeadDim];
-  __shared__ float part_s[4][G][4];  // m, l, D (1024 * sum of P), Z (sum of p * zero)
+__global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(uint16_t *o, const uint16_t *q, KvLayout c,
+                                                                              int num_qo_heads, float sm_scale_log2) {
+  __shared__ float part_o[kDecodeWaves][G][kHeadDim];
+  __shared__ float part_s[kDecodeWaves][G][4];  // m, l, D (1024 * sum of P), Z (sum of p * zero)
   const int b = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, g = lane >> 4;
@@ -398,9 +399,10 @@ __global__ __launch_bounds__(256) void kv_decode_i4_mfma_kernel(uint16_t *o, con
   const int len = np > 0 ? (np - 1) * c.page_size + c.last_page_offset[b] : 0;
   constexpr float kNegBig = -1e30f;
 
-  // Q^T operand: lane (head r16, group g) holds dims 32g + 8m + e for MFMA m, odd e divided by 16
+  // Q^T operand: lane (head r16, group g) holds dims 32g + 8m + kDimOfElem[e] for MFMA m, the
+  // elements of odd dims (high nibbles) divided by 16
   v8h qop[4];
-  float qsum = 0.0f;
+  float qsum = 0.0f, qoff = 0.0f;
   {
     const bool real = r16 < G;
     const uint16_t *qrow = q + ((size_t)b * num_qo_heads + h * G + (real ? r16 : 0)) * kHeadDim + 32 * g;
@@ -410,15 +412,20 @@ __global__ __launch_bounds__(256) void kv_decode_i4_mfma_kernel(uint16_t *o, con
       const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        float f = from_bits<BF16>(w[e >> 1] >> (16 * (e & 1)));
+        const int dim = kDimOfElem[e];
+        float f = from_bits<BF16>(w[dim >> 1] >> (16 * (dim & 1)));
         if (!real) f = 0.0f;
         const _Float16 hq = (_Float16)f;                 // exact for bf16 inputs inside the fp16 range
+        const _Float16 hs = (dim & 1) ? hq * (_Float16)0.0625f : hq;
         qsum += (float)hq;
-        qop[m][e] = (e & 1) ? hq * (_Float16)0.0625f : hq;
+        qoff += 1024.0f * (float)hs;                     // what the 1024 of this element's codes adds to a score
+        qop[m][e] = hs;
       }
     }
     qsum += __shfl_xor(qsum, 16);
     qsum += __shfl_xor(qsum, 32);
+    qoff += __shfl_xor(qoff, 16);
+    qoff += __shfl_xor(qoff, 32);
   }
 
   float m_run = kNegBig, l_run = 0.0f, d_run = 0.0f, z_run = 0.0f;
@@ -427,7 +434,7 @@ __global__ __launch_bounds__(256) void kv_decode_i4_mfma_kernel(uint16_t *o, con
   for (int j = 0; j < 8; ++j) oacc[j] = v4f{0.f, 0.f, 0.f, 0.f};
 
   const int nchunks = (len + 15) >> 4;
-  for (int ch = wave; ch < nchunks; ch += 4) {
+  for (int ch = wave; ch < nchunks; ch += kDecodeWaves) {
     const int t0 = ch << 4;
     const int page = c.indices[p0 + t0 / c.page_size], slot0 = t0 % c.page_size;
     const size_t krow0 = kv_row(c, page, 0, h, slot0), vrow0 = kv_row(c, page, 1, h, slot0);
@@ -451,7 +458,7 @@ __global__ __launch_bounds__(256) void kv_decode_i4_mfma_kernel(uint16_t *o, con
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const float ks = from_bits<BF16>(kp[v]), kz = from_bits<BF16>(kp[v] >> 16);
-      sc[v] = (t0 + 4 * g + v < len) ? (ks * sacc[v] - kz * qsum) * sm_scale_log2 : kNegBig;
+      sc[v] = (t0 + 4 * g + v < len) ? (ks * (sacc[v] - qoff) - kz * qsum) * sm_scale_log2 : kNegBig;
       mx = fmaxf(mx, sc[v]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16));
@@ -486,9 +493,8 @@ __global__ __launch_bounds__(256) void kv_decode_i4_mfma_kernel(uint16_t *o, con
     // V operands: byte bb of the four token dwords -> codes 2bb (low nibbles) and 2bb+1 (high nibbles)
 #define ARCQ_PV(BB)                                                                                             \
   {                                                                                                             \
-    const uint32_t x01 = __builtin_amdgcn_perm(vd[1], vd[0], 0x0c0c0400u + 0x00000101u * (BB));                 \
-    const uint32_t x23 = __builtin_amdgcn_perm(vd[3], vd[2], 0x0c0c0400u + 0x00000101u * (BB));                 \
-    const uint32_t t01 = __builtin_amdgcn_perm(0u, x01, 0x0c010c00u), t23 = __builtin_amdgcn_perm(0u, x23, 0x0c010c00u); \
+    const uint32_t t01 = __builtin_amdgcn_perm(vd[1], vd[0], 0x0c040c00u + 0x00010001u * (BB));                 \
+    const uint32_t t23 = __builtin_amdgcn_perm(vd[3], vd[2], 0x0c040c00u + 0x00010001u * (BB));                 \
     v2u lo, hi;                                                                                                 \
     lo[0] = (t01 & 0x000f000fu) | 0x64006400u;                                                                  \
     lo[1] = (t23 & 0x000f000fu) | 0x64006400u;                                                                  \
@@ -502,7 +508,7 @@ __global__ __launch_bounds__(256) void kv_decode_i4_mfma_kernel(uint16_t *o, con
 #undef ARCQ_PV
   }
 
-  // per-wave totals of the softmax sums over the four lane groups, then merge the four waves
+  // per-wave totals of the softmax sums over the four lane groups, then merge the waves
   l_run += __shfl_xor(l_run, 16);
   l_run += __shfl_xor(l_run, 32);
   d_run += __shfl_xor(d_run, 16);
@@ -522,15 +528,15 @@ __global__ __launch_bounds__(256) void kv_decode_i4_mfma_kernel(uint16_t *o, con
       for (int v = 0; v < G; ++v) part_o[wave][v][8 * r16 + j] = oacc[j][v];   // rows 4g+v = heads, g == 0
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < G * kHeadDim; idx += 256) {
+  for (int idx = threadIdx.x; idx < G * kHeadDim; idx += 64 * kDecodeWaves) {
     const int hh = idx / kHeadDim, dim = idx - hh * kHeadDim;
     float M = kNegBig;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) M = fmaxf(M, part_s[w][hh][0]);
+    for (int w = 0; w < kDecodeWaves; ++w) M = fmaxf(M, part_s[w][hh][0]);
     const float unscale = (dim & 1) ? 0.0625f : 1.0f;  // odd dims were accumulated as 16 n
     float num = 0.0f, den = 0.0f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < kDecodeWaves; ++w) {
       const float wgt = __builtin_amdgcn_exp2f(part_s[w][hh][0] - M);
       num = __builtin_fmaf(wgt, (part_o[w][hh][dim] - part_s[w][hh][2]) * unscale - part_s[w][hh][3], num);
       den = __builtin_fmaf(wgt, part_s[w][hh][1], den);
@@ -671,7 +677,8 @@ int arcq_kv_decode_i4(void *o, const void *q, int dtype, int batch, int num_qo_h
 #define ARCQ_LAUNCH_DECODE(BF, GG)                                                                                \
   do {                                                                                                            \
     if (mfma)                                                                                                     \
-      hipLaunchKernelGGL((kv_decode_i4_mfma_kernel<BF, GG>), grid, dim3(256), 0, st, op, qp, c, num_qo_heads, sl2); \
+      hipLaunchKernelGGL((kv_decode_i4_mfma_kernel<BF, GG>), grid, dim3(64 * kDecodeWaves), 0, st, op, qp, c,    \
+                         num_qo_heads, sl2);                                                                      \
     else                                                                                                          \
       hipLaunchKernelGGL((kv_decode_i4_kernel<BF, GG>), grid, dim3(256), 0, st, op, qp, c, num_qo_heads, sl2);    \
   } while (0)
