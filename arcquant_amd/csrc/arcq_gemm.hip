@@ -704,8 +704,8 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
 
 // ---------------------------------------------------------------------------------------------
 // Skinny kernels for M <= 64 (decode batches): the GEMM is a stream of the weight matrix, read
-// exactly once, so nothing is staged through LDS.  A workgroup owns 16 weight rows; its four waves
-// take the K steps of 128 round-robin in pairs (split-K: wave w does steps 2w, 2w+1, 2w+8, 2w+9, ...:
+// exactly once, so nothing is staged through LDS.  A workgroup owns 16 weight rows; its NW waves
+// take the K steps of 128 round-robin in pairs (split-K: with four waves wave w does steps 2w, 2w+1, 2w+8, 2w+9, ...:
 // a pair of steps is one whole 128-byte line of every row, and the four waves walk neighbouring lines) and their partial sums meet in LDS.  A lane loads
 // the 16 bytes (32 codes) the 16x16 MFMA wants from it straight from global memory: row lane%16,
 // K group lane/16, i.e. 64 contiguous bytes per row and step.  The activations (<= 64 rows) come
@@ -714,7 +714,7 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
 // ---------------------------------------------------------------------------------------------
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <int MT, int AT>
+template <int MT, int AT, int NW>
 __device__ __forceinline__ void skinny_reduce_store(const GemmParams &p, v4f (&acc)[AT * MT], float (*red)[MT * AT][64][4],
                                                     int wave, int lane) {
   if (wave > 0) {
@@ -731,7 +731,7 @@ __device__ __forceinline__ void skinny_reduce_store(const GemmParams &p, v4f (&a
     for (int j = 0; j < MT; ++j) {
       v4f t = acc[i * MT + j];
 #pragma unroll
-      for (int w = 0; w < 3; ++w) t += *reinterpret_cast<const v4f *>(red[w][i * MT + j][lane]);
+      for (int w = 0; w < NW - 1; ++w) t += *reinterpret_cast<const v4f *>(red[w][i * MT + j][lane]);
       const int m = 16 * j + (lane & 15);
       if (m >= p.M) continue;
       uint16_t *dst = p.c + (size_t)m * p.N + n0;
@@ -748,9 +748,9 @@ __device__ __forceinline__ void skinny_reduce_store(const GemmParams &p, v4f (&a
   }
 }
 
-template <int MT, int AT>
-__global__ __launch_bounds__(256) void gemm_mxfp4_skinny(GemmParams p) {
-  __shared__ float red[3][MT * AT][64][4];
+template <int MT, int AT, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_mxfp4_skinny(GemmParams p) {
+  __shared__ float red[NW - 1][MT * AT][64][4];
   constexpr int D = (MT * AT >= 4) ? 4 : 8;  // K steps whose loads are in flight together
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -773,12 +773,12 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_skinny(GemmParams p) {
 #pragma unroll
   for (int j = 0; j < AT * MT; ++j) acc[j] = v4f{0.f, 0.f, 0.f, 0.f};
   const uint32_t sh = 8u * (uint32_t)g;
-  for (int t0 = 2 * wave; t0 < T; t0 += 4 * D) {
+  for (int t0 = 2 * wave; t0 < T; t0 += NW * D) {
     uint4 a[AT][D], b[MT][D];
     uint32_t sa[AT][D], sb[MT][D];
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      const int t = t0 + 8 * (d >> 1) + (d & 1);
+      const int t = t0 + 2 * NW * (d >> 1) + (d & 1);
       if (t < T) {  // uniform over the wave
 #pragma unroll
         for (int i = 0; i < AT; ++i) {
@@ -794,7 +794,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_skinny(GemmParams p) {
     }
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      if (t0 + 8 * (d >> 1) + (d & 1) < T) {
+      if (t0 + 2 * NW * (d >> 1) + (d & 1) < T) {
 #pragma unroll
         for (int i = 0; i < AT; ++i)
 #pragma unroll
@@ -805,15 +805,15 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_skinny(GemmParams p) {
       }
     }
   }
-  skinny_reduce_store<MT, AT>(p, acc, red, wave, lane);
+  skinny_reduce_store<MT, AT, NW>(p, acc, red, wave, lane);
 }
 
 // NVFP4: the same walk; a lane's 16 bytes are two blocks of 16, decoded to fp16 eight codes at a
 // time and fed to four v_mfma_f32_16x16x32_f16.  Which K index a lane supplies to which of the four
 // is free as long as both operands agree: here MFMA d of a step takes K = 128t + 32*(lane/16) + 8d..+7.
-template <int MT>
-__global__ __launch_bounds__(256) void gemm_nvfp4_skinny(GemmParams p) {
-  __shared__ float red[3][MT][64][4];
+template <int MT, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_nvfp4_skinny(GemmParams p) {
+  __shared__ float red[NW - 1][MT][64][4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int T = p.Kp >> 7;
@@ -832,12 +832,12 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_skinny(GemmParams p) {
 #pragma unroll
   for (int j = 0; j < MT; ++j) acc[j] = v4f{0.f, 0.f, 0.f, 0.f};
   constexpr int D = MT >= 4 ? 2 : 4;  // K steps whose loads are in flight together
-  for (int t0 = 2 * wave; t0 < T; t0 += 4 * D) {
+  for (int t0 = 2 * wave; t0 < T; t0 += NW * D) {
     uint4 aq[D], bq[MT][D];
     uint32_t as2[D], bs2[MT][D];
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      const int t = t0 + 8 * (d >> 1) + (d & 1);
+      const int t = t0 + 2 * NW * (d >> 1) + (d & 1);
       if (t < T) {  // uniform over the wave
         aq[d] = *reinterpret_cast<const uint4 *>(wc + 64 * t);
         as2[d] = *reinterpret_cast<const uint16_t *>(ws + 8 * t);
@@ -850,7 +850,7 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_skinny(GemmParams p) {
     }
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      if (t0 + 8 * (d >> 1) + (d & 1) < T) {
+      if (t0 + 2 * NW * (d >> 1) + (d & 1) < T) {
         const uint32_t ap = nv_scale_pair_f16((as2[d] & 0xffu) | ((as2[d] & 0xff00u) << 8));
         const v8h a0 = decode8_nvfp4_f16<false>(aq[d].x, ap), a1 = decode8_nvfp4_f16<false>(aq[d].y, ap);
         const v8h a2 = decode8_nvfp4_f16<true>(aq[d].z, ap), a3 = decode8_nvfp4_f16<true>(aq[d].w, ap);
@@ -866,16 +866,26 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_skinny(GemmParams p) {
       }
     }
   }
-  skinny_reduce_store<MT, 1>(p, acc, red, wave, lane);
+  skinny_reduce_store<MT, 1, NW>(p, acc, red, wave, lane);
 }
 
+// NW waves per workgroup split K among them: eight where the layer is narrow (few workgroups, one wave
+// per SIMD otherwise), four where the grid alone fills the machine
 template <int FMT, int MT, int AT>
 int launch_skinny(const GemmParams &p, hipStream_t st) {
   const int grid = (p.N + 16 * AT - 1) / (16 * AT);
-  if (FMT == ARCQ_FMT_MXFP4)
-    hipLaunchKernelGGL((gemm_mxfp4_skinny<MT, AT>), dim3(grid), dim3(256), 0, st, p);
-  else
-    hipLaunchKernelGGL((gemm_nvfp4_skinny<MT>), dim3(grid), dim3(256), 0, st, p);
+  const bool eight = grid <= 512 && AT == 1;
+  if (FMT == ARCQ_FMT_MXFP4) {
+    if (eight)
+      hipLaunchKernelGGL((gemm_mxfp4_skinny<MT, 1, 8>), dim3(grid), dim3(512), 0, st, p);
+    else
+      hipLaunchKernelGGL((gemm_mxfp4_skinny<MT, AT, 4>), dim3(grid), dim3(256), 0, st, p);
+  } else {
+    if (eight)
+      hipLaunchKernelGGL((gemm_nvfp4_skinny<MT, 8>), dim3(grid), dim3(512), 0, st, p);
+    else
+      hipLaunchKernelGGL((gemm_nvfp4_skinny<MT, 4>), dim3(grid), dim3(256), 0, st, p);
+  }
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }
