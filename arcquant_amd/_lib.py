@@ -73,3 +73,41 @@ def lib() -> ctypes.CDLL:
 def check(status: int, where: str) -> None:
     if status != 0:
         raise ArcqError(status, where)
+
+
+# ------------------------------------------------------------------------------------------
+# launch plumbing shared by the operator modules: torch is asked for the current stream and the
+# current device through its cheapest entry points, since a decode step is a chain of launches
+# of a few microseconds each and the host must keep ahead of them
+# ------------------------------------------------------------------------------------------
+GROUP_SIZE = {NVFP4: 16, MXFP4: 32}
+
+
+def stream_of(t) -> ctypes.c_void_p:
+    """torch's current stream on t's device, as the `void *stream` of the C ABI"""
+    import torch
+    try:
+        return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(t.device.index))
+    except AttributeError:                       # a torch without the raw-stream hook
+        return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+class on_device_of:
+    """`with on_device_of(t):` makes t's device current for the launch; free when it already is"""
+    __slots__ = ("idx", "prev")
+
+    def __init__(self, t):
+        self.idx = t.device.index
+
+    def __enter__(self):
+        import torch
+        self.prev = torch.cuda.current_device()
+        if self.prev != self.idx:
+            torch.cuda.set_device(self.idx)
+
+    def __exit__(self, *exc):
+        if self.prev != self.idx:
+            import torch
+            torch.cuda.set_device(self.prev)
+        return False
+

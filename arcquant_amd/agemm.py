@@ -42,8 +42,8 @@ def _fmt_id(fmt) -> int:
         raise RuntimeError(f"unknown quantization format {fmt!r} (expected 'NVFP4' or 'MXFP4')") from None
 
 
-def _stream(t: torch.Tensor) -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+_stream = _lib.stream_of
+_on_device = _lib.on_device_of
 
 
 def _require(t: torch.Tensor, name: str, dtype, ndim=None):
@@ -68,6 +68,8 @@ def _scalar(value, device):
         if value.numel() != 1:
             raise RuntimeError("scale must be a scalar")
         if value.is_cuda:
+            if value.dtype == torch.float32 and value.device == device:
+                return 1.0, ctypes.c_void_p(value.data_ptr()), value
             v = value.detach().to(device=device, dtype=torch.float32).reshape(1)
             return 1.0, ctypes.c_void_p(v.data_ptr()), v
         return float(value), None, None
@@ -85,14 +87,14 @@ def _quantize(entry, X, gamma, eps, reorder_index, KE, fmt, global_scale):
     if reorder_index.device != X.device:
         raise RuntimeError("reorder_index must be on the same device as X")
     KE = int(KE)
-    G = L.arcq_group_size(f)
+    G = _lib.GROUP_SIZE[f]
     if K % 32 or K < 32 or K > 32736 or KE < 0 or KE > K or KE % G:
         raise RuntimeError(f"Value error in {entry}: K={K}, KE={KE} not supported for {fmt} "
                            f"(need K % 32 == 0, 32 <= K <= 32736, KE % {G} == 0, KE <= K)")
     gs, d_gs, keep = _scalar(global_scale, X.device)
     QX = torch.empty((M, (K + KE) // 2), dtype=torch.uint8, device=X.device)
-    SFX = torch.empty((L.arcq_scales_bytes(M, K, KE, f),), dtype=torch.uint8, device=X.device)
-    with torch.cuda.device(X.device):
+    SFX = torch.empty((M * ((K + KE) // G),), dtype=torch.uint8, device=X.device)
+    with _on_device(X):
         if gamma is None:
             rc = getattr(L, entry)(X.data_ptr(), M, K, reorder_index.data_ptr(), KE, f, gs, d_gs, QX.data_ptr(),
                                    SFX.data_ptr(), _stream(X))
@@ -135,7 +137,7 @@ def tensor_scale(x, divisor=2688.0):
     if K % 8 or ld % 8 or x.data_ptr() % 16:
         raise RuntimeError(f"Value error in tensor_scale: K={K}, row stride {ld} not supported")
     out = torch.empty((), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         rc = _lib.lib().arcq_tensor_scale(x.data_ptr(), None, ld, M, K, float(divisor), out.data_ptr(), _stream(x))
     _lib.check(rc, "arcq_tensor_scale")
     return out
@@ -161,11 +163,11 @@ def swiglu_quantize_x(gate, up, reorder_index, KE, *, fmt="NVFP4", global_scale=
     M, K = gate.shape
     ld = gate.stride(0) if M > 1 else K
     KE = int(KE)
-    G = L.arcq_group_size(f)
+    G = _lib.GROUP_SIZE[f]
     if K % 32 or K < 32 or K > 16384 or KE < 0 or KE > K or KE % G or reorder_index.numel() != K or ld % 8:
         raise RuntimeError(f"Value error in swiglu_quantize_x: K={K}, KE={KE}, row stride {ld} not supported for {fmt}")
     want_scale = isinstance(global_scale, str)
-    with torch.cuda.device(gate.device):
+    with _on_device(gate):
         if want_scale:
             if global_scale != "absmax":
                 raise RuntimeError("global_scale must be a number, a tensor or 'absmax'")
@@ -174,7 +176,7 @@ def swiglu_quantize_x(gate, up, reorder_index, KE, *, fmt="NVFP4", global_scale=
                                            _stream(gate)), "arcq_tensor_scale")
         gs, d_gs, keep = _scalar(global_scale, gate.device)
         QX = torch.empty((M, (K + KE) // 2), dtype=torch.uint8, device=gate.device)
-        SFX = torch.empty((L.arcq_scales_bytes(M, K, KE, f),), dtype=torch.uint8, device=gate.device)
+        SFX = torch.empty((M * ((K + KE) // G),), dtype=torch.uint8, device=gate.device)
         rc = L.arcq_swiglu_quantize_x(gate.data_ptr(), up.data_ptr(), ld, M, K, reorder_index.data_ptr(), KE, f, gs,
                                       d_gs, QX.data_ptr(), SFX.data_ptr(), _stream(gate))
     _lib.check(rc, "arcq_swiglu_quantize_x")
@@ -211,7 +213,7 @@ def matmul(A, B, SFA, SFB, scale, *, fmt=None):
     f = _infer_fmt(A, SFA, fmt)
     L = _lib.lib()
     M, N, Kp = A.shape[0], B.shape[0], 2 * A.shape[1]
-    G = L.arcq_group_size(f)
+    G = _lib.GROUP_SIZE[f]
     if SFA.numel() != M * (Kp // G) or SFB.numel() != N * (Kp // G):
         raise RuntimeError("scale buffers do not match the code buffers")
     if Kp % 64:
@@ -225,7 +227,7 @@ def matmul(A, B, SFA, SFB, scale, *, fmt=None):
         alpha, da, ka = _scalar(scale, A.device)
         db, kb = None, None
     C = torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
-    with torch.cuda.device(A.device):
+    with _on_device(A):
         rc = L.arcq_matmul(A.data_ptr(), SFA.data_ptr(), B.data_ptr(), SFB.data_ptr(), M, N, Kp, f, alpha, da, db,
                            C.data_ptr(), _stream(A))
     _lib.check(rc, "arcq_matmul")
@@ -244,7 +246,7 @@ def dequantize(Q, SF, *, fmt):
     _require(SF, "SF", torch.uint8)
     rows, Kp = Q.shape[0], 2 * Q.shape[1]
     out = torch.empty((rows, Kp), dtype=torch.float32, device=Q.device)
-    with torch.cuda.device(Q.device):
+    with _on_device(Q):
         rc = _lib.lib().arcq_dequantize(Q.data_ptr(), SF.data_ptr(), rows, Kp, f, out.data_ptr(), _stream(Q))
     _lib.check(rc, "arcq_dequantize")
     return out
@@ -253,7 +255,7 @@ def dequantize(Q, SF, *, fmt):
 def check_index(reorder_index) -> None:
     """Raises RuntimeError unless reorder_index (int16, CUDA) is a permutation of 0..K-1."""
     _require(reorder_index, "reorder_index", torch.int16, 1)
-    with torch.cuda.device(reorder_index.device):
+    with _on_device(reorder_index):
         rc = _lib.lib().arcq_check_index(reorder_index.data_ptr(), reorder_index.numel(), _stream(reorder_index))
     _lib.check(rc, "arcq_check_index")
 

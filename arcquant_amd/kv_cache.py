@@ -28,8 +28,7 @@ from . import _lib
 _DTYPES = {torch.float16: 0, torch.bfloat16: 1}
 
 
-def _stream(t):
-    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+_stream = _lib.stream_of
 
 
 def _ptr(t):
@@ -73,7 +72,7 @@ def quantize_append(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, 
         max_new_tokens = 1
     elif max_new_tokens is None:
         max_new_tokens = int(k.shape[0])
-    with torch.cuda.device(k.device):
+    with _lib.on_device_of(k):
         rc = _lib.lib().arcq_kv_append_i4(_ptr(k), _ptr(v), _DTYPES[k.dtype], batch, _ptr(seqlen_indptr),
                                           int(max_new_tokens), _ptr(kv_data), _ptr(kv_param), _ptr(kv_indptr),
                                           _ptr(kv_indices), _ptr(last_page_offset), n_layers, int(layer_idx), heads,
@@ -109,7 +108,7 @@ def rope_quantize_append(qkv, num_qo_heads, cos_table, sin_table, positions, kv_
         raise RuntimeError("positions must be an int32 CUDA tensor [batch]")
     if q_out is None:
         q_out = torch.empty(batch, num_qo_heads, head_dim, dtype=qkv.dtype, device=qkv.device)
-    with torch.cuda.device(qkv.device):
+    with _lib.on_device_of(qkv):
         rc = _lib.lib().arcq_rope_kv_append_i4(_ptr(qkv), int(qkv.stride(0)), _DTYPES[qkv.dtype], batch,
                                                int(num_qo_heads), _ptr(cos_table), _ptr(sin_table),
                                                int(cos_table.shape[0]), _ptr(positions), _ptr(q_out), _ptr(kv_data),
@@ -133,7 +132,7 @@ def _store(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_p
     k, v, k_param, v_param = (t.contiguous() for t in (k, v, k_param, v_param))
     batch = last_page_offset.numel()
     max_new = 1 if seqlen_indptr is None else int(k.shape[0])
-    with torch.cuda.device(k.device):
+    with _lib.on_device_of(k):
         rc = _lib.lib().arcq_kv_store_i4(_ptr(k), _ptr(v), _ptr(k_param), _ptr(v_param), batch, _ptr(seqlen_indptr),
                                          max_new, _ptr(kv_data), _ptr(kv_param), _ptr(kv_indptr), _ptr(kv_indices),
                                          _ptr(last_page_offset), n_layers, int(layer_idx), heads, page_size, head_dim,
@@ -163,7 +162,7 @@ def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_of
         raise RuntimeError("q / o must be contiguous with the cache's head_dim")
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(head_dim)
-    with torch.cuda.device(q.device):
+    with _lib.on_device_of(q):
         rc = _lib.lib().arcq_kv_decode_i4(_ptr(o), _ptr(q), _DTYPES[q.dtype], q.shape[0], q.shape[1], _ptr(kv_data),
                                           _ptr(kv_param), _ptr(kv_indptr), _ptr(kv_indices), _ptr(last_page_offset),
                                           n_layers, int(layer_idx), heads, page_size, head_dim, float(sm_scale),
