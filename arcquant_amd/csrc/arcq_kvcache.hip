@@ -18,6 +18,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "../../include/arcq.h"
 #include "arcq_internal.h"
 #include "arcq_math.h"
@@ -387,9 +389,14 @@ __device__ __forceinline__ v8h k_operand(uint32_t x) {
 // MFMAs), so the kernel lives on waves per SIMD, and batch x KV heads workgroups of four waves give
 // only two.
 constexpr int kDecodeWaves = 8;
+// With few sequences the (sequence, KV head) grid leaves CUs idle: gridDim.z > 1 cuts every sequence's
+// chunks into that many ranges, one workgroup each, which write (maximum, denominator, numerator[128])
+// per head to `partial` instead of the output; kv_decode_merge_kernel combines them.
+constexpr int kPartialStride = kHeadDim + 2;
 template <bool BF16, int G>
 __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(uint16_t *o, const uint16_t *q, KvLayout c,
-                                                                              int num_qo_heads, float sm_scale_log2) {
+                                                                              int num_qo_heads, float sm_scale_log2,
+                                                                              float *partial) {
   __shared__ float part_o[kDecodeWaves][G][kHeadDim];
   __shared__ float part_s[kDecodeWaves][G][4];  // m, l, D (1024 * sum of P), Z (sum of p * zero)
   const int b = blockIdx.x, h = blockIdx.y;
@@ -434,7 +441,8 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(ui
   for (int j = 0; j < 8; ++j) oacc[j] = v4f{0.f, 0.f, 0.f, 0.f};
 
   const int nchunks = (len + 15) >> 4;
-  for (int ch = wave; ch < nchunks; ch += kDecodeWaves) {
+  const int ch_beg = (int)((long)nchunks * blockIdx.z / gridDim.z), ch_end = (int)((long)nchunks * (blockIdx.z + 1) / gridDim.z);
+  for (int ch = ch_beg + wave; ch < ch_end; ch += kDecodeWaves) {
     const int t0 = ch << 4;
     const int page = c.indices[p0 + t0 / c.page_size], slot0 = t0 % c.page_size;
     const size_t krow0 = kv_row(c, page, 0, h, slot0), vrow0 = kv_row(c, page, 1, h, slot0);
@@ -541,9 +549,53 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(ui
       num = __builtin_fmaf(wgt, (part_o[w][hh][dim] - part_s[w][hh][2]) * unscale - part_s[w][hh][3], num);
       den = __builtin_fmaf(wgt, part_s[w][hh][1], den);
     }
+    if (gridDim.z > 1) {
+      float *dst = partial + (((size_t)b * num_qo_heads + h * G + hh) * gridDim.z + blockIdx.z) * kPartialStride;
+      dst[2 + dim] = num;
+      if (dim == 0) {
+        dst[0] = M;
+        dst[1] = den;
+      }
+      continue;
+    }
     const float out = den > 0.0f ? num / den : 0.0f;
     o[((size_t)b * num_qo_heads + h * G + hh) * kHeadDim + dim] = (uint16_t)to_bits<BF16>(out);
   }
+}
+
+// one workgroup of 128 threads per (sequence, query head): softmax-weighted sum of the ranges' partials
+template <bool BF16>
+__global__ __launch_bounds__(128) void kv_decode_merge_kernel(uint16_t *o, const float *partial, int splits) {
+  const float *src = partial + (size_t)blockIdx.x * splits * kPartialStride;
+  float M = -1e30f;
+  for (int z = 0; z < splits; ++z) M = fmaxf(M, src[z * kPartialStride]);
+  float num = 0.0f, den = 0.0f;
+  for (int z = 0; z < splits; ++z) {
+    const float wgt = __builtin_amdgcn_exp2f(src[z * kPartialStride] - M);
+    num = __builtin_fmaf(wgt, src[z * kPartialStride + 2 + threadIdx.x], num);
+    den = __builtin_fmaf(wgt, src[z * kPartialStride + 1], den);
+  }
+  const float out = den > 0.0f ? num / den : 0.0f;
+  o[(size_t)blockIdx.x * kHeadDim + threadIdx.x] = (uint16_t)to_bits<BF16>(out);
+}
+
+// partials of the split decode: one buffer per device, allocated on first use and kept
+constexpr size_t kDecodeWorkspaceBytes = 8u << 20;
+inline float *decode_workspace() {
+  static std::mutex mu;
+  static float *ws[16];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ws[dev]) {
+    float *w = nullptr;
+    if (hipMalloc(&w, kDecodeWorkspaceBytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    ws[dev] = w;
+  }
+  return ws[dev];
 }
 
 int check_layout(const void *kv_data, const void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
@@ -668,19 +720,35 @@ int arcq_kv_decode_i4(void *o, const void *q, int dtype, int batch, int num_qo_h
              num_kv_heads,
              page_size};
   const float sl2 = sm_scale * 1.4426950408889634f;
-  dim3 grid(batch, num_kv_heads);
+  static const bool force_valu = getenv("ARCQ_KV_DECODE_VALU") != nullptr;
+  static const int split_env = getenv("ARCQ_KV_DECODE_SPLITS") ? atoi(getenv("ARCQ_KV_DECODE_SPLITS")) : 0;
+  const bool mfma = page_size % 16 == 0 && !force_valu;
+  // few (sequence, KV head) pairs: cut the sequences so that about two workgroups per CU exist (the
+  // lengths live on the device, so the cut is by count only; a range without tokens costs nothing)
+  int splits = 1;
+  float *partial = nullptr;
+  if (mfma) {
+    const long pairs = (long)batch * num_kv_heads;
+    splits = split_env > 0 ? split_env : (pairs >= 256 ? 1 : (int)((512 + pairs - 1) / pairs));
+    if (splits > 16) splits = 16;
+    if (splits > 1) {
+      partial = decode_workspace();
+      if (!partial || (size_t)batch * num_qo_heads * splits * kPartialStride * sizeof(float) > kDecodeWorkspaceBytes)
+        splits = 1;
+    }
+  }
+  dim3 grid(batch, num_kv_heads, splits);
   hipStream_t st = static_cast<hipStream_t>(stream);
   uint16_t *op = static_cast<uint16_t *>(o);
   const uint16_t *qp = static_cast<const uint16_t *>(q);
-  static const bool force_valu = getenv("ARCQ_KV_DECODE_VALU") != nullptr;
-  const bool mfma = page_size % 16 == 0 && !force_valu;
 #define ARCQ_LAUNCH_DECODE(BF, GG)                                                                                \
   do {                                                                                                            \
     if (mfma)                                                                                                     \
       hipLaunchKernelGGL((kv_decode_i4_mfma_kernel<BF, GG>), grid, dim3(64 * kDecodeWaves), 0, st, op, qp, c,    \
-                         num_qo_heads, sl2);                                                                      \
+                         num_qo_heads, sl2, partial);                                                             \
     else                                                                                                          \
-      hipLaunchKernelGGL((kv_decode_i4_kernel<BF, GG>), grid, dim3(256), 0, st, op, qp, c, num_qo_heads, sl2);    \
+      hipLaunchKernelGGL((kv_decode_i4_kernel<BF, GG>), dim3(batch, num_kv_heads), dim3(256), 0, st, op, qp, c,  \
+                         num_qo_heads, sl2);                                                                      \
   } while (0)
   if (dtype == ARCQ_DTYPE_BF16) {
     if (G == 1) ARCQ_LAUNCH_DECODE(true, 1);
@@ -693,6 +761,13 @@ int arcq_kv_decode_i4(void *o, const void *q, int dtype, int batch, int num_qo_h
   }
 #undef ARCQ_LAUNCH_DECODE
   ARCQ_HIP_TRY(hipGetLastError());
+  if (splits > 1) {
+    if (dtype == ARCQ_DTYPE_BF16)
+      hipLaunchKernelGGL(kv_decode_merge_kernel<true>, dim3(batch * num_qo_heads), dim3(128), 0, st, op, partial, splits);
+    else
+      hipLaunchKernelGGL(kv_decode_merge_kernel<false>, dim3(batch * num_qo_heads), dim3(128), 0, st, op, partial, splits);
+    ARCQ_HIP_TRY(hipGetLastError());
+  }
   return ARCQ_OK;
 }
 

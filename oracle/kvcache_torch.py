@@ -34,6 +34,10 @@ def gather_sequence(pages, params, indptr, indices, last_page_offset, layer, b):
     ids = indices[indptr[b]:indptr[b + 1]].tolist()
     n = (len(ids) - 1) * page_size + int(last_page_offset[b]) if ids else 0
     out = []
+    if not ids:                                    # a sequence without pages
+        heads = pages.shape[3]
+        empty = (torch.zeros(0, heads, 128, dtype=torch.uint8), torch.zeros(0, heads, 2, dtype=torch.float64))
+        return [empty, empty]
     for kv in (0, 1):
         codes = torch.cat([unpack(pages[p, layer, kv]) for p in ids], dim=1)[:, :n]       # [heads, len, 128]
         par = torch.cat([params[p, layer, kv] for p in ids], dim=1)[:, :n].double()        # [heads, len, 2]

@@ -207,3 +207,32 @@ def test_rope_quantize_append_is_bit_exact(kvc, ref, dtype):
             assert torch.equal(codes[-1:], ref.unpack(qq))
             assert torch.equal(par[-1:, :, 0], s[..., 0].double()) and torch.equal(par[-1:, :, 1], z[..., 0].double())
             assert int(codes[:-1].sum()) == 0                # earlier slots untouched
+
+
+def test_decode_attention_many_sequences(kvc, ref):
+    """Enough (sequence, KV head) pairs that the kernel takes every sequence whole (one workgroup per
+    pair, no split ranges, no merge launch); the small batches above take the split path.  One sequence
+    is empty: its output is zero."""
+    batch, q_heads, kv_heads, page_size, dtype = 40, 32, 8, 16, torch.bfloat16
+    g = torch.Generator().manual_seed(17)
+    lengths = [int(n) for n in torch.randint(1, 90, (batch,), generator=g)]
+    lengths[7] = 0
+    total = sum(lengths)
+    k = torch.randn(total, kv_heads, 128, generator=g).to(dtype)
+    v = torch.randn(total, kv_heads, 128, generator=g).to(dtype)
+    q = torch.randn(batch, q_heads, 128, generator=g).to(dtype)
+    indptr, indices, last, maxc = make_table(lengths, page_size, batch)
+    pages = torch.zeros(maxc * batch, 1, 2, kv_heads, page_size, 64, dtype=torch.uint8, device="cuda")
+    params = torch.full((maxc * batch, 1, 2, kv_heads, page_size, 2), float("nan"), dtype=dtype, device="cuda")
+    offs = [0]
+    for n in lengths:
+        offs.append(offs[-1] + n)
+    print("kv decode, 40 sequences x 8 KV heads", flush=True)
+    kvc.quantize_append(pages, params, indptr.cuda(), indices.cuda(), last.cuda(), k.cuda(), v.cuda(), 0,
+                        seqlen_indptr=torch.tensor(offs, dtype=torch.int32).cuda(), max_new_tokens=max(lengths))
+    o = torch.full_like(q, 7.0).cuda()
+    kvc.batch_decode_i4(o, q.cuda(), pages, params, indptr.cuda(), indices.cuda(), last.cuda(), 0)
+    want = ref.decode_attention(q, pages.cpu(), params.cpu(), indptr, indices, last, 0)
+    keep = [b for b in range(batch) if b != 7]
+    assert rel_fro(o[keep], want[keep]) < 5e-3
+    assert float(o[7].abs().sum()) == 0.0
