@@ -56,6 +56,7 @@ def lib() -> ctypes.CDLL:
     L.arcq_tensor_scale.argtypes = [vp, vp, i, i, i, f, vp, vp]
     L.arcq_kv_append_i4.argtypes = [vp, vp, i, i, vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
     L.arcq_rope_kv_append_i4.argtypes = [vp, i, i, i, i, vp, vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
+    L.arcq_rope.argtypes = [vp, i, i, ctypes.c_long, i, i, i, i, i, vp, vp, i, vp, vp, vp]
     L.arcq_kv_store_i4.argtypes = [vp, vp, vp, vp, i, vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
     L.arcq_kv_decode_i4.argtypes = [vp, vp, i, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, f, vp]
     L.arcq_matmul.argtypes = [vp, vp, vp, vp, i, i, i, i, f, vp, vp, vp, vp]

@@ -18,6 +18,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <algorithm>
 #include <mutex>
 
 #include "../../include/arcq.h"
@@ -182,6 +183,46 @@ __global__ __launch_bounds__(256) void rope_kv_append_i4_kernel(const uint16_t *
       const int head = r - num_qo_heads - kv * c.heads;
       quantize_values_store<BF16>(x, c, kv_row(c, page, kv, head, slot), lane16);
     }
+  }
+}
+
+// the rotary embedding alone, for whole prompts: token t of the flattened [sequences x q_len] batch sits
+// at position pos0 + t % q_len; rotated query heads go to q_out [tokens, query heads, 128], rotated key
+// heads to k_out [tokens, kv heads, 128] (the value heads stay where they are)
+template <bool BF16>
+__global__ __launch_bounds__(256) void rope_rows_kernel(const uint16_t *qkv, int ld, const uint16_t *cos_t,
+                                                        const uint16_t *sin_t, int max_positions, int q_len, int pos0,
+                                                        long rows_total, int num_qo_heads, int num_kv_heads,
+                                                        uint16_t *q_out, uint16_t *k_out) {
+  const int lane16 = threadIdx.x & 15;
+  const int heads = num_qo_heads + num_kv_heads;
+  for (long row = (long)blockIdx.x * 16 + (threadIdx.x >> 4); row < rows_total; row += (long)gridDim.x * 16) {
+    const long tok = row / heads;
+    const int head = (int)(row - tok * heads);
+    const int pos = min(max(pos0 + (int)(tok % q_len), 0), max_positions - 1);
+    const uint4 raw = reinterpret_cast<const uint4 *>(qkv + (size_t)tok * ld + (size_t)head * kHeadDim)[lane16];
+    float x[8], xp[8], cs[8], sn[8];
+    unpack8<BF16>(raw, x);
+    uint4 praw;
+    praw.x = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)raw.x, 0x128, 0xf, 0xf, true);  // row_ror:8 = lane ^ 8
+    praw.y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)raw.y, 0x128, 0xf, 0xf, true);
+    praw.z = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)raw.z, 0x128, 0xf, 0xf, true);
+    praw.w = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)raw.w, 0x128, 0xf, 0xf, true);
+    unpack8<BF16>(praw, xp);
+    const size_t t = (size_t)pos * (kHeadDim / 2) + 8 * (lane16 & 7);
+    unpack8<BF16>(*reinterpret_cast<const uint4 *>(cos_t + t), cs);
+    unpack8<BF16>(*reinterpret_cast<const uint4 *>(sin_t + t), sn);
+    const float sgn = lane16 < 8 ? -1.0f : 1.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = rn<BF16>(rn<BF16>(x[i] * cs[i]) + rn<BF16>((sgn * xp[i]) * sn[i]));
+    uint4 o;
+    o.x = to_bits<BF16>(x[0]) | (to_bits<BF16>(x[1]) << 16);
+    o.y = to_bits<BF16>(x[2]) | (to_bits<BF16>(x[3]) << 16);
+    o.z = to_bits<BF16>(x[4]) | (to_bits<BF16>(x[5]) << 16);
+    o.w = to_bits<BF16>(x[6]) | (to_bits<BF16>(x[7]) << 16);
+    uint16_t *dst = head < num_qo_heads ? q_out + ((size_t)tok * num_qo_heads + head) * kHeadDim
+                                        : k_out + ((size_t)tok * num_kv_heads + (head - num_qo_heads)) * kHeadDim;
+    reinterpret_cast<uint4 *>(dst)[lane16] = o;
   }
 }
 
@@ -668,6 +709,36 @@ int arcq_rope_kv_append_i4(const void *qkv, int ld, int dtype, int batch, int nu
     hipLaunchKernelGGL(rope_kv_append_i4_kernel<false>, grid, dim3(256), 0, st, static_cast<const uint16_t *>(qkv), ld,
                        static_cast<const uint16_t *>(cos_table), static_cast<const uint16_t *>(sin_table), max_positions,
                        positions, static_cast<uint16_t *>(q_out), num_qo_heads, c);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+int arcq_rope(const void *qkv, int ld, int dtype, long tokens, int q_len, int pos0, int num_qo_heads, int num_kv_heads,
+              int head_dim, const void *cos_table, const void *sin_table, int max_positions, void *q_out, void *k_out,
+              void *stream) {
+  using namespace arcq;
+  if (dtype != ARCQ_DTYPE_F16 && dtype != ARCQ_DTYPE_BF16) return ARCQ_ERR_FORMAT;
+  const long heads = (long)num_qo_heads + num_kv_heads;
+  if (head_dim != kHeadDim || tokens < 0 || q_len < 1 || num_qo_heads < 1 || num_kv_heads < 0 || max_positions < 1 ||
+      ld < heads * kHeadDim || ld % 8 != 0)
+    return ARCQ_ERR_SHAPE;
+  if (tokens == 0) return ARCQ_OK;
+  if (!qkv || !cos_table || !sin_table || !q_out || (num_kv_heads > 0 && !k_out)) return ARCQ_ERR_NULL;
+  if (!aligned16(qkv) || !aligned16(cos_table) || !aligned16(sin_table) || !aligned16(q_out) || !aligned16(k_out))
+    return ARCQ_ERR_ALIGN;
+  const long rows = tokens * heads;
+  const unsigned grid = (unsigned)std::min<long>((rows + 15) / 16, 16384);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ARCQ_DTYPE_BF16)
+    hipLaunchKernelGGL(rope_rows_kernel<true>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(qkv), ld,
+                       static_cast<const uint16_t *>(cos_table), static_cast<const uint16_t *>(sin_table), max_positions,
+                       q_len, pos0, rows, num_qo_heads, num_kv_heads, static_cast<uint16_t *>(q_out),
+                       static_cast<uint16_t *>(k_out));
+  else
+    hipLaunchKernelGGL(rope_rows_kernel<false>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(qkv), ld,
+                       static_cast<const uint16_t *>(cos_table), static_cast<const uint16_t *>(sin_table), max_positions,
+                       q_len, pos0, rows, num_qo_heads, num_kv_heads, static_cast<uint16_t *>(q_out),
+                       static_cast<uint16_t *>(k_out));
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }

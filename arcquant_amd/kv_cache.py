@@ -88,6 +88,30 @@ def rope_tables(max_positions, head_dim, dtype, device, base=10000.0):
     return freqs.cos().to(dtype).contiguous(), freqs.sin().to(dtype).contiguous()
 
 
+def rope(qkv, q_len, pos0, num_qo_heads, num_kv_heads, cos_table, sin_table):
+    """Rotary embedding of the query and key heads of a fused qkv projection output [tokens, (q + 2 kv
+    heads) * 128] (rows may be strided); token t sits at position pos0 + t % q_len.  Returns the rotated
+    q [tokens, num_qo_heads, 128] and k [tokens, num_kv_heads, 128]; same values as torch's
+    q * cos + rotate_half(q) * sin in qkv's dtype (model/qLlamaLayer.py:30-64)."""
+    if qkv.dim() != 2 or qkv.dtype not in _DTYPES or qkv.stride(1) != 1 or not qkv.is_cuda:
+        raise RuntimeError("qkv must be a 2-D fp16 / bf16 CUDA tensor with unit stride along its last dimension")
+    tokens = qkv.shape[0]
+    if qkv.shape[1] < (num_qo_heads + 2 * num_kv_heads) * 128 or tokens % q_len:
+        raise RuntimeError("qkv does not match the head counts or q_len")
+    for t in (cos_table, sin_table):
+        if t.dtype != qkv.dtype or t.dim() != 2 or t.shape[1] != 64 or not t.is_contiguous():
+            raise RuntimeError("cos / sin tables must be contiguous [positions, 64] of qkv's dtype")
+    q = torch.empty(tokens, num_qo_heads, 128, dtype=qkv.dtype, device=qkv.device)
+    k = torch.empty(tokens, num_kv_heads, 128, dtype=qkv.dtype, device=qkv.device)
+    ld = qkv.stride(0) if tokens > 1 else qkv.shape[1]
+    with _lib.on_device_of(qkv):
+        rc = _lib.lib().arcq_rope(_ptr(qkv), int(ld), _DTYPES[qkv.dtype], tokens, int(q_len), int(pos0),
+                                  int(num_qo_heads), int(num_kv_heads), 128, _ptr(cos_table), _ptr(sin_table),
+                                  int(cos_table.shape[0]), _ptr(q), _ptr(k), _stream(qkv))
+    _lib.check(rc, "arcq_rope")
+    return q, k
+
+
 def rope_quantize_append(qkv, num_qo_heads, cos_table, sin_table, positions, kv_data, kv_param, kv_indptr, kv_indices,
                          last_page_offset, layer_idx, q_out=None):
     """One decode step between the qkv projection and the attention (model/qLlamaLayer.py:316-327):

@@ -34,6 +34,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import agemm
+from . import kv_cache as _kvc
 
 NVFP4_RANGE = 448.0 * 6.0   # model/qLlamaLayer.py:74
 
@@ -224,6 +225,7 @@ class LlamaAttention(nn.Module):
         self.o_proj = QLinearLayer(o, select_num_o, o_index, quant_type=quant_type)
         self.register_buffer("o_reorder_index", o_index.to(torch.int16))
         self.quant_type = quant_type
+        self._rope = None                    # cos / sin tables of the fused rotary embedding, built on first use
 
     @torch.no_grad()
     def forward(self, x, kv_cache=None, past_len=0, layer_idx=0):
@@ -239,10 +241,20 @@ class LlamaAttention(nn.Module):
             # decode over the INT4 pages: rotary embedding + quantized append in one launch, then attention
             out = kv_cache.decode_step(qkv.view(bsz, -1), nh, layer_idx).view(bsz, 1, nh * d)
             return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num, self.quant_type))
-        q = qkv[..., :nh * d].view(bsz, q_len, nh, d).transpose(1, 2)
-        k = qkv[..., nh * d:(nh + nkv) * d].view(bsz, q_len, nkv, d).transpose(1, 2)
         v = qkv[..., (nh + nkv) * d:].view(bsz, q_len, nkv, d).transpose(1, 2)
-        q, k = rotary_pos_emb(q, k, past_len)
+        if isinstance(past_len, int) and d == 128:
+            # rotary embedding of q and k in one pass over the projection output (same values as
+            # rotary_pos_emb below: every product and the sum rounded to bf16)
+            need = past_len + q_len
+            if self._rope is None or self._rope[0].shape[0] < need:
+                self._rope = _kvc.rope_tables(max(need, 4096), d, qkv.dtype, qkv.device)
+            q, k = _kvc.rope(qkv.view(bsz * q_len, -1), q_len, past_len, nh, nkv, *self._rope)
+            q = q.view(bsz, q_len, nh, d).transpose(1, 2)
+            k = k.view(bsz, q_len, nkv, d).transpose(1, 2)
+        else:
+            q = qkv[..., :nh * d].view(bsz, q_len, nh, d).transpose(1, 2)
+            k = qkv[..., nh * d:(nh + nkv) * d].view(bsz, q_len, nkv, d).transpose(1, 2)
+            q, k = rotary_pos_emb(q, k, past_len)
         if kv_cache is not None and not isinstance(kv_cache, tuple):
             r = kv_cache.update(k.transpose(1, 2), v.transpose(1, 2), layer_idx)
             if callable(r):                                   # decode: attention over the INT4 pages

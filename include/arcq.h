@@ -195,6 +195,16 @@ int arcq_rope_kv_append_i4(const void *qkv, int ld, int dtype, int batch, int nu
                            void *kv_data, void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
                            const int32_t *last_page_offset, int n_layers, int layer_idx, int num_kv_heads, int page_size,
                            int head_dim, void *stream);
+/*
+ * The rotary embedding alone, for prompts (apply_rotary_pos_emb, model/qLlamaLayer.py:30-64, evaluated as
+ * torch does on tensors of the model dtype): token t of the flattened [sequences x q_len] batch sits at
+ * position pos0 + t % q_len.  qkv [tokens, ld] as above; the rotated query heads go to q_out
+ * [tokens, num_qo_heads, 128] and the rotated key heads to k_out [tokens, num_kv_heads, 128]; the value
+ * heads are not touched.  One pass over q and k instead of torch's six.
+ */
+int arcq_rope(const void *qkv, int ld, int dtype, long tokens, int q_len, int pos0, int num_qo_heads, int num_kv_heads,
+              int head_dim, const void *cos_table, const void *sin_table, int max_positions, void *q_out, void *k_out,
+              void *stream);
 /* the same scatter for rows the caller has quantized already -- the exact argument set of the
  * reference's init_kv_i4 (seqlen_indptr given) and append_kv_i4 (seqlen_indptr NULL):
  * k_codes / v_codes u8 [tokens, kv_heads, 64], k_param / v_param [tokens, kv_heads, 2] */

@@ -236,3 +236,25 @@ def test_decode_attention_many_sequences(kvc, ref):
     keep = [b for b in range(batch) if b != 7]
     assert rel_fro(o[keep], want[keep]) < 5e-3
     assert float(o[7].abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_rows_match_torch(kvc, dtype):
+    """The one-pass rotary embedding of a prompt against torch's q * cos + rotate_half(q) * sin on the
+    CPU (every op rounded to the dtype): bit-identical, for strided projection rows and a start offset."""
+    seqs, q_len, nh, nkv, pos0 = 3, 21, 4, 2, 5
+    g = torch.Generator().manual_seed(23)
+    width = (nh + 2 * nkv) * 128
+    wide = (torch.randn(seqs * q_len, width + 8, generator=g) * 2).to(dtype)
+    cos_t, sin_t = kvc.rope_tables(64, 128, dtype, "cuda")
+    print(f"rope rows {dtype}", flush=True)
+    q_rot, k_rot = kvc.rope(wide.cuda()[:, :width], q_len, pos0, nh, nkv, cos_t, sin_t)
+    torch.cuda.synchronize()
+    pos = (pos0 + torch.arange(seqs * q_len) % q_len).long()
+    cos = torch.cat([cos_t.cpu(), cos_t.cpu()], dim=-1)[pos][:, None]
+    sin = torch.cat([sin_t.cpu(), sin_t.cpu()], dim=-1)[pos][:, None]
+    rot = lambda x: torch.cat((-x[..., 64:], x[..., :64]), dim=-1)
+    q = wide[:, :nh * 128].view(-1, nh, 128)
+    k = wide[:, nh * 128:(nh + nkv) * 128].view(-1, nkv, 128)
+    assert torch.equal(q_rot.cpu(), q * cos + rot(q) * sin)
+    assert torch.equal(k_rot.cpu(), k * cos + rot(k) * sin)
