@@ -347,9 +347,22 @@ __device__ __forceinline__ void unit_exact(const uint32_t (&yv)[16], float g, ui
 // act_fn(gate) * up as the reference's layers form it in bf16 (model/qLlamaLayer.py:432,
 // model/qMixtralLayer.py:531): SiLU evaluated in fp32 as x / (1 + exp(-x)) and rounded to bf16,
 // then a bf16 multiply (fp32 product, one rounding).  Two elements per call, packed.
-__device__ __forceinline__ uint32_t swiglu_pair(uint32_t gw, uint32_t uw) {
+// The SiLU of a bf16 value has only 65536 possible inputs: the hardware estimates
+// x * rcp(1 + exp2(-x * log2 e)) round to the same bf16 as the library expression for every one of them
+// except 5.9375 and -87.5, -88, -88.5 (all 65536 inputs compared on the GPU; a test repeats it).  Waves
+// that hold one of those, anything of magnitude >= 87, or a NaN take the library expression.
+__device__ __forceinline__ uint32_t silu_pair_bf16(uint32_t gw) {
   const float g0 = u2f(gw << 16), g1 = u2f(gw & 0xffff0000u);
-  const uint32_t a = pack_bf16_rne(g0 / (1.0f + expf(-g0)), g1 / (1.0f + expf(-g1)));
+  const uint32_t m0 = gw & 0x7fffu, m1 = (gw >> 16) & 0x7fffu;
+  const bool special = m0 >= 0x42aeu || m1 >= 0x42aeu || (gw & 0xffffu) == 0x40beu || (gw >> 16) == 0x40beu;
+  if (__builtin_amdgcn_ballot_w64(special) != 0)
+    return pack_bf16_rne(g0 / (1.0f + expf(-g0)), g1 / (1.0f + expf(-g1)));
+  const float e0 = __builtin_amdgcn_exp2f(g0 * -1.4426950408889634f), e1 = __builtin_amdgcn_exp2f(g1 * -1.4426950408889634f);
+  return pack_bf16_rne(g0 * __builtin_amdgcn_rcpf(1.0f + e0), g1 * __builtin_amdgcn_rcpf(1.0f + e1));
+}
+
+__device__ __forceinline__ uint32_t swiglu_pair(uint32_t gw, uint32_t uw) {
+  const uint32_t a = silu_pair_bf16(gw);
   return pack_bf16_rne(dot2_bf16(a, uw & 0xffffu), dot2_bf16(a, uw & 0xffff0000u));
 }
 

@@ -74,3 +74,33 @@ def test_errors(agemm):
         agemm.swiglu_quantize_x(g.float(), g.float(), idx, 0)
     with pytest.raises(RuntimeError):
         agemm.swiglu_quantize_x(g, g, idx, 16, fmt="MXFP4")     # select_num not a multiple of 32
+
+
+def test_silu_of_every_bf16_value(agemm):
+    """The SiLU inside the fused kernels against torch's own bf16 silu on the GPU for all 65536 bf16
+    inputs: arcq_tensor_scale over a tensor of eight copies of g with up = 1 and divisor 1 returns
+    |silu(g)| itself.  Finite inputs only: the kernels form the product with `up` through a two-term dot
+    product whose unused term is x * 0, which turns an infinite x into NaN."""
+    import ctypes
+    from arcquant_amd import _lib
+    L = _lib.lib()
+    bits = torch.arange(65536, dtype=torch.int32)
+    g = (bits << 16).view(torch.float32).to(torch.bfloat16)          # exact: the low half is zero
+    finite = torch.isfinite(g.float())
+    gate = g.cuda()[:, None].repeat(1, 8).contiguous()               # [65536, 8]
+    up = torch.ones(8, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(65536, dtype=torch.float32, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    print("silu over all bf16 values", flush=True)
+    base_g, base_o = gate.data_ptr(), out.data_ptr()
+    for i in range(65536):
+        if not bool(finite[i]):
+            continue
+        rc = L.arcq_tensor_scale(base_g + 16 * i, up.data_ptr(), 8, 1, 8, 1.0, base_o + 4 * i, stream)
+        assert rc == 0
+    torch.cuda.synchronize()
+    want = F.silu(g.cuda()).abs().float()
+    want = torch.where(want == 0, torch.ones_like(want), want)       # the entry point maps an all-zero tensor to 1
+    got, want = out.cpu()[finite], want.cpu()[finite]
+    bad = (got != want).nonzero().flatten()
+    assert bad.numel() == 0, [(hex(int(bits[finite][j])), float(got[j]), float(want[j])) for j in bad[:8]]
