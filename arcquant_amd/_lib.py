@@ -60,6 +60,7 @@ def lib() -> ctypes.CDLL:
     L.arcq_kv_store_i4.argtypes = [vp, vp, vp, vp, i, vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
     L.arcq_kv_decode_i4.argtypes = [vp, vp, i, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, f, vp]
     L.arcq_matmul.argtypes = [vp, vp, vp, vp, i, i, i, i, f, vp, vp, vp, vp]
+    L.arcq_matmul_add.argtypes = [vp, vp, vp, vp, i, i, i, i, f, vp, vp, vp, vp, vp]
     L.arcq_check_index.argtypes = [vp, i, vp]
     L.arcq_dequantize.argtypes = [vp, vp, i, i, i, vp, vp]
     L.arcq_stream_probe.argtypes = [vp, vp, sz, sz, vp]

@@ -196,13 +196,14 @@ def _infer_fmt(A, SFA, fmt):
     raise RuntimeError(f"cannot tell the block format from SFA ({n} scale bytes for {M}x{2 * half} values)")
 
 
-def matmul(A, B, SFA, SFB, scale, *, fmt=None):
+def matmul(A, B, SFA, SFB, scale, *, fmt=None, residual=None):
     """agemm.matmul (kernels/src/bindings.cpp:99-120): bf16 [M,N] = scale * dq(A) @ dq(B)^T.
 
     A u8 [M,K'/2], B u8 [N,K'/2], SFA/SFB as returned by the quantizers.  ``scale`` may be a
     python float (as in the reference), a 0-dim tensor, or a pair of 0-dim CUDA tensors
     (scale_x, scale_w) whose product is formed on the device -- the last two avoid the host sync
-    the reference's float argument forces (model/qLinearLayer.py:69).
+    the reference's float argument forces (model/qLinearLayer.py:69).  ``residual`` bf16 [M,N]: added
+    in the epilogue, with the result of ``matmul(...) + residual`` bit for bit.
     """
     _require(A, "A", torch.uint8, 2)
     _require(B, "B", torch.uint8, 2)
@@ -228,8 +229,15 @@ def matmul(A, B, SFA, SFB, scale, *, fmt=None):
         db, kb = None, None
     C = torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
     with _on_device(A):
-        rc = L.arcq_matmul(A.data_ptr(), SFA.data_ptr(), B.data_ptr(), SFB.data_ptr(), M, N, Kp, f, alpha, da, db,
-                           C.data_ptr(), _stream(A))
+        if residual is None:
+            rc = L.arcq_matmul(A.data_ptr(), SFA.data_ptr(), B.data_ptr(), SFB.data_ptr(), M, N, Kp, f, alpha, da, db,
+                               C.data_ptr(), _stream(A))
+        else:
+            _require(residual, "residual", torch.bfloat16, 2)
+            if tuple(residual.shape) != (M, N) or residual.device != A.device:
+                raise RuntimeError(f"residual must be bf16 [{M}, {N}] on A's device")
+            rc = L.arcq_matmul_add(A.data_ptr(), SFA.data_ptr(), B.data_ptr(), SFB.data_ptr(), M, N, Kp, f, alpha, da,
+                                   db, residual.data_ptr(), C.data_ptr(), _stream(A))
     _lib.check(rc, "arcq_matmul")
     del ka, kb
     return C

@@ -38,7 +38,20 @@ struct GemmParams {
   // writes its fp32 partial tile to partial[slice][M][N] instead of C; splitk_reduce_kernel adds them
   float *partial = nullptr;
   int k_slices = 1;
+  // optional residual, bf16 [M,N]: C = bf16(bf16(alpha * acc) + residual), what a bf16 add of the
+  // rounded GEMM output and the residual gives
+  const uint16_t *residual = nullptr;
 };
+
+// two bf16 pairs + two bf16 pairs, each sum rounded to bf16
+__device__ __forceinline__ uint32_t add_bf16_pair(uint32_t a, uint32_t b) {
+  const uint32_t lo = f32_to_bf16_bits(bf16_bits_to_f32(a & 0xffffu) + bf16_bits_to_f32(b & 0xffffu));
+  const uint32_t hi = f32_to_bf16_bits(bf16_bits_to_f32(a >> 16) + bf16_bits_to_f32(b >> 16));
+  return lo | (hi << 16);
+}
+__device__ __forceinline__ uint2 add_bf16_x4(uint2 a, uint2 b) {
+  return make_uint2(add_bf16_pair(a.x, b.x), add_bf16_pair(a.y, b.y));
+}
 
 __device__ __forceinline__ float effective_alpha(const GemmParams &p) {
   float a = p.alpha;
@@ -62,7 +75,9 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, const v16f &acc,
       uint32_t h[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) h[j] = f32_to_bf16_bits(acc[4 * q + j] * alpha);
-      *reinterpret_cast<uint2 *>(crow + 8 * q) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+      uint2 v = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+      if (p.residual) v = add_bf16_x4(v, *reinterpret_cast<const uint2 *>(p.residual + (crow - p.c) + 8 * q));
+      *reinterpret_cast<uint2 *>(crow + 8 * q) = v;
     }
     return;
   }
@@ -74,6 +89,12 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, const v16f &acc,
     uint32_t h[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) h[j] = f32_to_bf16_bits(acc[4 * q + j] * alpha);
+    if (p.residual) {
+      const uint16_t *rrow = p.residual + (size_t)m * p.N;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n + j < p.N) h[j] = f32_to_bf16_bits(bf16_bits_to_f32(h[j]) + bf16_bits_to_f32(rrow[n + j]));
+    }
     if (n + 3 < p.N && (p.N & 3) == 0) {
       *reinterpret_cast<uint2 *>(crow + n) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
     } else {
@@ -299,7 +320,12 @@ __device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (
     for (int it = 0; it < (32 * WM * LPR) / 64; ++it) {
       const int m = it * (64 / LPR) + rr;
       const int sw = (m & (LPR - 1)) << 1;
-      const uint4 v = *reinterpret_cast<const uint4 *>(region + m * RB + (((2 * t) ^ sw) << 3));
+      uint4 v = *reinterpret_cast<const uint4 *>(region + m * RB + (((2 * t) ^ sw) << 3));
+      if (p.residual) {
+        const uint4 rv = *reinterpret_cast<const uint4 *>(p.residual + (cbase - p.c) + (size_t)m * p.N);
+        v = make_uint4(add_bf16_pair(v.x, rv.x), add_bf16_pair(v.y, rv.y), add_bf16_pair(v.z, rv.z),
+                       add_bf16_pair(v.w, rv.w));
+      }
       *reinterpret_cast<uint4 *>(cbase + (size_t)m * p.N) = v;
     }
     return;
@@ -738,11 +764,17 @@ __device__ __forceinline__ void skinny_reduce_store(const GemmParams &p, v4f (&a
       if (n0 + 3 < p.N && (p.N & 3) == 0) {
         const uint32_t lo = f32_to_bf16_bits(t[0] * alpha) | (f32_to_bf16_bits(t[1] * alpha) << 16);
         const uint32_t hi = f32_to_bf16_bits(t[2] * alpha) | (f32_to_bf16_bits(t[3] * alpha) << 16);
-        *reinterpret_cast<uint2 *>(dst) = make_uint2(lo, hi);
+        uint2 v = make_uint2(lo, hi);
+        if (p.residual) v = add_bf16_x4(v, *reinterpret_cast<const uint2 *>(p.residual + (dst - p.c)));
+        *reinterpret_cast<uint2 *>(dst) = v;
       } else {
 #pragma unroll
         for (int v = 0; v < 4; ++v)
-          if (n0 + v < p.N) dst[v] = (uint16_t)f32_to_bf16_bits(t[v] * alpha);
+          if (n0 + v < p.N) {
+            uint32_t hb = f32_to_bf16_bits(t[v] * alpha);
+            if (p.residual) hb = f32_to_bf16_bits(bf16_bits_to_f32(hb) + bf16_bits_to_f32(p.residual[(dst - p.c) + v]));
+            dst[v] = (uint16_t)hb;
+          }
       }
     }
   }
@@ -936,7 +968,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p) {
     }
     const uint32_t lo = f32_to_bf16_bits(t.x * alpha) | (f32_to_bf16_bits(t.y * alpha) << 16);
     const uint32_t hi = f32_to_bf16_bits(t.z * alpha) | (f32_to_bf16_bits(t.w * alpha) << 16);
-    reinterpret_cast<uint2 *>(p.c)[i] = make_uint2(lo, hi);
+    uint2 v = make_uint2(lo, hi);
+    if (p.residual) v = add_bf16_x4(v, reinterpret_cast<const uint2 *>(p.residual)[i]);
+    reinterpret_cast<uint2 *>(p.c)[i] = v;
   }
 }
 
@@ -979,9 +1013,27 @@ int launch_tiled_splitk(GemmParams p, int slices, hipStream_t st) {
 }  // namespace
 }  // namespace arcq
 
+static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
+                       int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b,
+                       const void *residual, void *c, void *stream);
+
 extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
                            int M, int N, int Kp, int fmt, float alpha, const float *d_alpha_a,
                            const float *d_alpha_b, void *c, void *stream) {
+  return matmul_impl(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b, nullptr, c, stream);
+}
+
+extern "C" int arcq_matmul_add(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                               int M, int N, int Kp, int fmt, float alpha, const float *d_alpha_a,
+                               const float *d_alpha_b, const void *residual, void *c, void *stream) {
+  if (!residual) return ARCQ_ERR_NULL;
+  if (!arcq::aligned16(residual)) return ARCQ_ERR_ALIGN;
+  return matmul_impl(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b, residual, c, stream);
+}
+
+static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
+                       int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b,
+                       const void *residual, void *c, void *stream) {
   using namespace arcq;
   if (fmt != ARCQ_FMT_NVFP4 && fmt != ARCQ_FMT_MXFP4) return ARCQ_ERR_FORMAT;
   if (M < 0 || N < 0 || Kp < 64 || Kp % 64 != 0) return ARCQ_ERR_SHAPE;
@@ -1000,6 +1052,7 @@ extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void
   p.M = M;
   p.N = N;
   p.Kp = Kp;
+  p.residual = static_cast<const uint16_t *>(residual);
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 grid((N + kWgN - 1) / kWgN, (M + kWgM - 1) / kWgM);
   // Tile choice (ARCQ_GEMM_KERNEL=<WN><WM> forces one, 0 forces the direct kernels; for tuning):

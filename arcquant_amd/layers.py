@@ -126,12 +126,18 @@ class QLinearLayer(nn.Module):
             self.bias = None
 
     @torch.no_grad()
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """residual [..., out_features]: added to the output (in the GEMM's epilogue when the layer has
+        no bias), same bits as `self(x) + residual`"""
         qx, scale_x, scale, bsz, q_len = x
         alpha = (scale, self.scale) if isinstance(scale, torch.Tensor) else (float(scale), self.scale)
-        y = agemm.matmul(qx, self.W, scale_x, self.scale_w, alpha, fmt=self.quant_type)
+        fused = residual is not None and self.bias is None
+        y = agemm.matmul(qx, self.W, scale_x, self.scale_w, alpha, fmt=self.quant_type,
+                         residual=residual.reshape(-1, self.out_features).contiguous() if fused else None)
         if self.bias is not None:
             y = y + self.bias
+        if residual is not None and not fused:
+            y = y + residual.reshape(-1, self.out_features)
         if bsz is not None:
             return y.reshape(bsz, q_len, -1)
         return y.reshape(q_len, -1)
@@ -202,14 +208,15 @@ class LlamaMLP(nn.Module):
         self.quant_type = quant_type
 
     @torch.no_grad()
-    def forward(self, x):
-        """x: the tuple of the already quantized (normalised) hidden states"""
+    def forward(self, x, residual=None):
+        """x: the tuple of the already quantized (normalised) hidden states; residual: added to the output"""
         gu = self.gate_up_proj(x)
         if self.inter <= 16384 and self.inter % 32 == 0:
             return self.down_proj(swiglu_quantize_tokens(gu, self.inter, self.down_reorder_index,
-                                                         self.down_proj.select_num, self.quant_type))
+                                                         self.down_proj.select_num, self.quant_type), residual)
         t = F.silu(gu[..., :self.inter]) * gu[..., self.inter:]
-        return self.down_proj(quantize_tokens(t, self.down_reorder_index, self.down_proj.select_num, self.quant_type))
+        return self.down_proj(quantize_tokens(t, self.down_reorder_index, self.down_proj.select_num, self.quant_type),
+                              residual)
 
 
 class LlamaAttention(nn.Module):
@@ -228,8 +235,8 @@ class LlamaAttention(nn.Module):
         self._rope = None                    # cos / sin tables of the fused rotary embedding, built on first use
 
     @torch.no_grad()
-    def forward(self, x, kv_cache=None, past_len=0, layer_idx=0):
-        """x: quantized hidden states (tuple).  kv_cache: None, or (k, v) bf16 [bsz, kv_heads, L, d]
+    def forward(self, x, kv_cache=None, past_len=0, layer_idx=0, residual=None):
+        """x: quantized hidden states (tuple); residual: added to the output.  kv_cache: None, or (k, v) bf16 [bsz, kv_heads, L, d]
         holding past_len valid positions (the new keys/values are written behind them), or an
         arcquant_amd.kv_cache.MultiLayerPagedKVCache4Bit (INT4 pages; decode attention then runs on
         the quantized cache, model/qLlamaLayer.py:334-338 with model/kv_cache.py:214-279)."""
@@ -240,7 +247,8 @@ class LlamaAttention(nn.Module):
                 not kv_cache._needs_init[layer_idx]:
             # decode over the INT4 pages: rotary embedding + quantized append in one launch, then attention
             out = kv_cache.decode_step(qkv.view(bsz, -1), nh, layer_idx).view(bsz, 1, nh * d)
-            return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num, self.quant_type))
+            return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num, self.quant_type),
+                               residual)
         v = qkv[..., (nh + nkv) * d:].view(bsz, q_len, nkv, d).transpose(1, 2)
         if isinstance(past_len, int) and d == 128:
             # rotary embedding of q and k in one pass over the projection output (same values as
@@ -260,7 +268,7 @@ class LlamaAttention(nn.Module):
             if callable(r):                                   # decode: attention over the INT4 pages
                 out = r(q.transpose(1, 2)).reshape(bsz, q_len, nh * d)
                 return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num,
-                                                   self.quant_type))
+                                                   self.quant_type), residual)
             kv_cache = None                                   # prefill: attend to the fresh keys / values
         if kv_cache is not None:
             kc, vc = kv_cache
@@ -270,7 +278,7 @@ class LlamaAttention(nn.Module):
         out = F.scaled_dot_product_attention(q, k, v, is_causal=(q_len > 1 and past_len == 0),
                                              enable_gqa=(nkv != nh))
         out = out.transpose(1, 2).reshape(bsz, q_len, nh * d)
-        return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num, self.quant_type))
+        return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num, self.quant_type), residual)
 
 
 class LlamaDecoderLayer(nn.Module):
@@ -305,8 +313,9 @@ class LlamaDecoderLayer(nn.Module):
 
     @torch.no_grad()
     def forward(self, hidden_states, kv_cache=None, past_len=0, layer_idx=0):
-        h = hidden_states + self.self_attn(self.input_layernorm(hidden_states), kv_cache, past_len, layer_idx)
-        return h + self.mlp(self.post_attention_layernorm(h))
+        # both residual adds happen in the epilogues of the o and down projections
+        h = self.self_attn(self.input_layernorm(hidden_states), kv_cache, past_len, layer_idx, residual=hidden_states)
+        return self.mlp(self.post_attention_layernorm(h), residual=h)
 
 
 class MixtralExpertMLP(nn.Module):

@@ -149,6 +149,16 @@ int arcq_matmul(const void *a_codes, const void *a_scales, const void *b_codes, 
                 void *stream);
 
 /*
+ * The same GEMM with a residual added in the epilogue: C = bf16(bf16(alpha * acc) + residual), residual
+ * bf16 [M,N] -- bit for bit what a bf16 add of arcq_matmul's output and the residual gives (the
+ * reference's layers add the attention / MLP output to the hidden states as a separate torch op,
+ * benchmarks/modeling_arc.py:318-328), without the output's round trip through memory.
+ */
+int arcq_matmul_add(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
+                    int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b, const void *residual,
+                    void *c, void *stream);
+
+/*
  * INT4 paged KV cache (the reference's decode-attention path: agemm.init_kv_i4 / append_kv_i4 /
  * batch_decode_i4, kernels/src/bindings.cpp:287-413 -> kernels/src/flashinfer.cu:9-112, with the
  * torch-side quantizer asym_quantize_and_pack_i4, model/kv_cache.py:23-37, fused into the append).

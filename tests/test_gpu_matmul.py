@@ -138,3 +138,27 @@ def test_matmul_decode_batches(agemm, fmt, M, N, K, S):
     y_big = agemm.matmul(a, b, sfa, sfb, gx * gw)[:M]
     # same operands, fp32 accumulation in another order, one bf16 rounding each
     assert rel_fro(y.float(), y_big.float()) < 4e-3
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("M,N,K,S", [
+    (1, 4096, 4096, 256),      # skinny, eight waves
+    (48, 6144, 4096, 256),     # split-K: the second launch adds
+    (64, 4100, 8192, 128),     # split-K with a ragged last tile
+    (33, 28672, 1024, 128),    # tiled 128x64
+    (300, 1000, 2048, 128),    # tiled, ragged M and N: transposed epilogue and the per-element one
+    (1100, 1024, 1024, 0),     # 256x256 tiles (MXFP4 cost model may take smaller ones) with a ragged M
+    (130, 384, 448, 64),       # K' % 128 != 0: direct kernels
+    (5, 202, 384, 0),          # N % 4 != 0: scalar stores
+])
+def test_matmul_with_residual_equals_separate_add(agemm, fmt, M, N, K, S):
+    """arcq_matmul_add through every epilogue: the same bits as matmul(...) + residual in bf16."""
+    (x, w, idx, gx, gw), (a, sfa, b, sfb) = quantized_pair(agemm, M, N, K, S, fmt, seed=90 + M)
+    g = torch.Generator().manual_seed(M * 7 + N)
+    r = (torch.randn(M, N, generator=g) * 0.7).to(torch.bfloat16).cuda()
+    print(f"matmul + residual {fmt} M={M} N={N} K={K} S={S}", flush=True)
+    y = agemm.matmul(a, b, sfa, sfb, gx * gw)
+    z = agemm.matmul(a, b, sfa, sfb, gx * gw, residual=r)
+    assert torch.equal(z, y + r)
+    with pytest.raises(RuntimeError):
+        agemm.matmul(a, b, sfa, sfb, gx * gw, residual=r[:, :-1].contiguous())
