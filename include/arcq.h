@@ -152,7 +152,7 @@ int arcq_matmul(const void *a_codes, const void *a_scales, const void *b_codes, 
  * The same GEMM with a residual added in the epilogue: C = bf16(bf16(alpha * acc) + residual), residual
  * bf16 [M,N] -- bit for bit what a bf16 add of arcq_matmul's output and the residual gives (the
  * reference's layers add the attention / MLP output to the hidden states as a separate torch op,
- * benchmarks/modeling_arc.py:318-328), without the output's round trip through memory.
+ * model/qLlamaLayer.py:147-168, benchmarks/modeling_arc.py:284-307), without the output's round trip through memory.
  */
 int arcq_matmul_add(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
                     int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b, const void *residual,
