@@ -251,6 +251,32 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, a), __builtin_bit_cast(v2bf, b), 0.0f, false);
 }
 
+// pack_bf16_rne(h_even * gamma_even, h_odd * gamma_odd) for four registers of bf16 pairs.  Written as
+// one block because the compiler only reaches the two-operand v_dot2c_f32_bf16 (a zeroed accumulator
+// register per product, then wait states in front of every conversion).  A dot instruction's result
+// may be read by another kind of VALU instruction only three issue slots later: each conversion
+// below has at least three instructions between it and the later of its two products, and nothing
+// outside the block can come closer than that to a product either.
+__device__ __forceinline__ void gamma_mul_pack4(const uint32_t *h, const uint32_t *glo, const uint32_t *ghi, uint32_t *out) {
+  float a0, a1, a2, a3, b0, b1, b2, b3;
+  asm("v_dot2_f32_bf16 %4, %12, %16, 0\n\t"
+      "v_dot2_f32_bf16 %8, %12, %20, 0\n\t"
+      "v_dot2_f32_bf16 %5, %13, %17, 0\n\t"
+      "v_dot2_f32_bf16 %9, %13, %21, 0\n\t"
+      "v_dot2_f32_bf16 %6, %14, %18, 0\n\t"
+      "v_dot2_f32_bf16 %10, %14, %22, 0\n\t"
+      "v_dot2_f32_bf16 %7, %15, %19, 0\n\t"
+      "v_dot2_f32_bf16 %11, %15, %23, 0\n\t"
+      "v_cvt_pk_bf16_f32 %0, %4, %8\n\t"
+      "v_cvt_pk_bf16_f32 %1, %5, %9\n\t"
+      "v_cvt_pk_bf16_f32 %2, %6, %10\n\t"
+      "v_cvt_pk_bf16_f32 %3, %7, %11"
+      : "=&v"(out[0]), "=&v"(out[1]), "=&v"(out[2]), "=&v"(out[3]), "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3),
+        "=&v"(b0), "=&v"(b1), "=&v"(b2), "=&v"(b3)
+      : "v"(h[0]), "v"(h[1]), "v"(h[2]), "v"(h[3]), "v"(glo[0]), "v"(glo[1]), "v"(glo[2]), "v"(glo[3]), "v"(ghi[0]),
+        "v"(ghi[1]), "v"(ghi[2]), "v"(ghi[3]));
+}
+
 // Sum of one double per lane over the 64 lanes of a wave, in DPP register moves (no LDS round
 // trips): prefix sums inside each row of 16 lanes, then the row totals are passed along.
 // The total ends up in lane 63.
@@ -492,12 +518,11 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
       } else {
         rstd = 1.0f / sqrtf(a);
       }
-      uint32_t yw[8];
+      uint32_t hw[8], yw[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t h = pack_bf16_rne(f[2 * j] * rstd, f[2 * j + 1] * rstd);
-        yw[j] = pack_bf16_rne(dot2_bf16(h, glo[j]), dot2_bf16(h, ghi[j]));
-      }
+      for (int j = 0; j < 8; ++j) hw[j] = pack_bf16_rne(f[2 * j] * rstd, f[2 * j + 1] * rstd);
+      gamma_mul_pack4(hw, glo, ghi, yw);
+      gamma_mul_pack4(hw + 4, glo + 4, ghi + 4, yw + 4);
       if (active) {
         reinterpret_cast<uint4 *>(row)[tid] = make_uint4(yw[0], yw[1], yw[2], yw[3]);
         reinterpret_cast<uint4 *>(row)[tid + nunits] = make_uint4(yw[4], yw[5], yw[6], yw[7]);
