@@ -468,7 +468,7 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
   for (int i = 0; i < 16; ++i) yv[i] = 0u;  // low halves stay zero: only d16_hi loads write these
 
   for (; r < p.rows; r += gridDim.x) {
-    uint4 n0 = q0, n1 = q1, un0 = u0, un1 = u1;
+    uint4 n0, n1, un0, un1;  // left undefined past the last row: nothing reads them then
     if (r + (int)gridDim.x < p.rows && active) {  // prefetch the next row of this workgroup
       const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)(r + gridDim.x) * ldx);
       n0 = src[tid];
@@ -604,15 +604,20 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
         sb2 = sb;
       }
     }
-    if (active) {
-      store_unit<FMT>(crow, srow, tid, pk, sb);
-      if (tail) store_unit<FMT>(crow, srow, nunits + (tid - tail0), pk2, sb2);
-    }
+    // The next row's registers are taken over before this row's stores are issued: the wait for
+    // the prefetch (in flight since the top of the iteration) then stands in front of the stores, and
+    // the top of the next iteration has no memory operation of this one left to wait for.
     q0 = n0;
     q1 = n1;
+    asm volatile("" : "+v"(q0.x), "+v"(q0.y), "+v"(q0.z), "+v"(q0.w), "+v"(q1.x), "+v"(q1.y), "+v"(q1.z), "+v"(q1.w));
     if (MODE == MODE_SWIGLU) {
       u0 = un0;
       u1 = un1;
+      asm volatile("" : "+v"(u0.x), "+v"(u0.y), "+v"(u0.z), "+v"(u0.w), "+v"(u1.x), "+v"(u1.y), "+v"(u1.z), "+v"(u1.w));
+    }
+    if (active) {
+      store_unit<FMT>(crow, srow, tid, pk, sb);
+      if (tail) store_unit<FMT>(crow, srow, nunits + (tid - tail0), pk2, sb2);
     }
   }
 }
