@@ -113,14 +113,16 @@ def test_matmul_llama_shapes_vs_torch_fp32(agemm, fmt, M, N, K, S):
 
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 32, 48, 64])
-@pytest.mark.parametrize("N,K,S", [(6144, 4096, 256), (202, 384, 0), (4100, 1024, 128), (4100, 8192, 128)])
+@pytest.mark.parametrize("N,K,S", [(6144, 4096, 256), (202, 384, 0), (4100, 1024, 128), (4100, 8192, 128),
+                                   (8324, 1024, 256), (8450, 768, 256)])
 def test_matmul_decode_batches(agemm, fmt, M, N, K, S):
     """M <= 64 (decode batches) at a benchmark shape and at shapes whose N is not a multiple of the
     16-row strips or of the 4-wide stores: against torch's fp32 matmul of the dequantized operands,
     and, row by row, against the same call on a 128-row batch that contains these rows (another
     kernel computes that one).  The long-K shape and the wider batches of the benchmark shape take the
     split-K path (partial tiles in a workspace, added by a second launch): a repeated call must give
-    the same bits."""
+    the same bits.  The two wide shapes take the 128x64 tiles with a ragged last workgroup, one of them
+    with N % 4 != 0."""
     (x, w, idx, gx, gw), (a, sfa, b, sfb) = quantized_pair(agemm, 128, N, K, S, fmt, seed=11)
     print(f"matmul decode {fmt} M={M} N={N} K={K} S={S}", flush=True)
     a_m = a[:M].contiguous()
@@ -146,6 +148,7 @@ def test_matmul_decode_batches(agemm, fmt, M, N, K, S):
     (48, 6144, 4096, 256),     # split-K: the second launch adds
     (64, 4100, 8192, 128),     # split-K with a ragged last tile
     (33, 28672, 1024, 128),    # tiled 128x64
+    (40, 8324, 1024, 256),     # tiled 128x64, ragged last workgroup
     (300, 1000, 2048, 128),    # tiled, ragged M and N: transposed epilogue and the per-element one
     (1100, 1024, 1024, 0),     # 256x256 tiles (MXFP4 cost model may take smaller ones) with a ragged M
     (130, 384, 448, 64),       # K' % 128 != 0: direct kernels
