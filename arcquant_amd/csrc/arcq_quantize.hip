@@ -246,8 +246,8 @@ __device__ __forceinline__ float scale_rcp(float s) {
 // gamma * h for the two bf16 halves of one register: v_dot2_f32_bf16 with the other half of the
 // gamma operand zeroed gives the exact fp32 product without unpacking h
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b) {
-  // the builtin, not inline asm: the compiler then sees the instruction and keeps the wait states
-  // it needs after the VALU instructions that produce its operands
+  // the builtin, not a bare inline-asm instruction: the compiler then sees a dot instruction and
+  // keeps the wait states its result needs before another kind of instruction may read it
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, a), __builtin_bit_cast(v2bf, b), 0.0f, false);
 }
 
@@ -256,10 +256,13 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b) {
 // register per product, then wait states in front of every conversion).  A dot instruction's result
 // may be read by another kind of VALU instruction only three issue slots later: each conversion
 // below has at least three instructions between it and the later of its two products, and nothing
-// outside the block can come closer than that to a product either.
+// outside the block can come closer than that to a product either.  The compiler does not know what
+// the block's instructions are, so the block also opens with the two wait states that cover every
+// forwarding hazard between a VALU instruction in front of it and a dot reading that result.
 __device__ __forceinline__ void gamma_mul_pack4(const uint32_t *h, const uint32_t *glo, const uint32_t *ghi, uint32_t *out) {
   float a0, a1, a2, a3, b0, b1, b2, b3;
-  asm("v_dot2_f32_bf16 %4, %12, %16, 0\n\t"
+  asm("s_nop 1\n\t"
+      "v_dot2_f32_bf16 %4, %12, %16, 0\n\t"
       "v_dot2_f32_bf16 %8, %12, %20, 0\n\t"
       "v_dot2_f32_bf16 %5, %13, %17, 0\n\t"
       "v_dot2_f32_bf16 %9, %13, %21, 0\n\t"

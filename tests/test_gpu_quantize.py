@@ -77,6 +77,24 @@ def test_rmsnorm_quantize_x(agemm, oracle, fmt, M, K, S):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
+def test_rmsnorm_quantize_x_benchmark_size(agemm, oracle, fmt):
+    """The benchmark's launch (4096 x 4096, select_num 256) against the oracle, every row, and the same
+    bits from every one of a series of back-to-back launches."""
+    M, K, S = 4096, 4096, 256
+    x = recipes.activations(M, K, seed=515, outlier_frac=0.005, outlier_gain=50.0)
+    gam = recipes.gamma(K, seed=8)
+    idx = recipes.reorder_index(x)
+    want = oracle.rmsnorm_quantize_x(x, gam, 1e-5, idx, S, fmt, 1.0)
+    print(f"rmsnorm_quantize_x {fmt} M={M} K={K} S={S}", flush=True)
+    xd, gd, idxd = dev(x), dev(gam), dev(idx)
+    q, sf = agemm.rmsnorm_quantize_x(xd, gd, 1e-5, idxd, S, fmt=fmt)
+    compare("rmsnorm 4096x4096", q, sf, want)
+    outs = [agemm.rmsnorm_quantize_x(xd, gd, 1e-5, idxd, S, fmt=fmt) for _ in range(12)]
+    for q2, sf2 in outs:
+        assert torch.equal(q2, q) and torch.equal(sf2, sf)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
 def test_edge_values(agemm, oracle, fmt):
     """zeros, ties, tiny and huge blocks, negative-only blocks, bf16 subnormals."""
     M, K = 8, 256
