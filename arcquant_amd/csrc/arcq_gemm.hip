@@ -343,11 +343,12 @@ __device__ __forceinline__ v8i fp4_operand(uint4 q) {
   return __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1);
 }
 
-template <int WN, int WM>
+template <int WN, int WM, int NS = 2>
 __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
   constexpr int BN = 64 * WN, BM = 64 * WM;
-  __shared__ uint4 sW[2 * BN * 8], sX[2 * BM * 8];  // code tiles, two stages each
-  __shared__ uint4 sWs[2 * BN], sXs[2 * BM];        // 16 scale bytes per row (two K steps), two stages each
+  static_assert(NS == 2 || (NS == 4 && WN == 2 && WM == 1), "the four-stage ring's wait counts are those of the 128x64 tile");
+  __shared__ uint4 sW[NS * BN * 8], sX[NS * BM * 8];  // code tiles, NS stages each
+  __shared__ uint4 sWs[NS * BN], sXs[NS * BM];        // 16 scale bytes per row (two K steps), NS stages each
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kbytes = p.Kp >> 1, ksc = p.Kp >> 5;
@@ -391,7 +392,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
   const uint32_t lxs0 = (uint32_t)reinterpret_cast<uintptr_t>(sXs);
 
   auto issue = [&](int kt) {
-    const int st = kt & 1;
+    const int st = kt & (NS - 1);
     // a short last step has only chunks 0..3: fetch those twice; the products of the absent blocks
     // are zeroed in compute()
     const bool clip = short_last && kt == nk - 1;
@@ -401,7 +402,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
 #pragma unroll
     for (int i = 0; i < WM * 2; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * 4096);
     if ((kt & 1) == 0) {  // scales of steps kt and kt+1
-      const int pair = kt >> 1, sst = pair & 1;
+      const int pair = kt >> 1, sst = pair & (NS - 1);
       const int soff = pair * 16 - (pair == npairs - 1 ? sc_shift : 0);
 #pragma unroll
       for (int j = 0; j < WN; ++j)
@@ -437,7 +438,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
   // sets), so LDS latency hides behind the matrix pipe.
   auto compute = [&](int kt, auto tail) {
     constexpr bool TAIL = decltype(tail)::value;
-    const int st = kt & 1, sst = (kt >> 1) & 1;
+    const int st = kt & (NS - 1), sst = (kt >> 1) & (NS - 1);
     const uint4 *cw = sW + st * (BN * 8), *cx = sX + st * (BM * 8);
     // this lane's four scale bytes of the step inside the row's 16-byte pair window; a lane whose
     // blocks are absent (short last step) may point past it and is clamped: its operands are zero
@@ -490,14 +491,34 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
   const int kt_end = min(nk, 2 * (int)((long)npairs * (blockIdx.y + 1) / p.k_slices));
   const bool tail = short_last && kt_end == nk;
   const int nfull = tail ? kt_end - 1 : kt_end;
-  if (kt_beg < kt_end) issue(kt_beg);
+  // NS - 1 steps are on their way while one is computed.  With two stages the wait for a step is a
+  // wait for everything; with four, the two younger steps stay outstanding: this wave issued 6 code
+  // loads for each of them and, for the even one of the two, its share of the scale loads (one
+  // instruction for waves 0..2, none for wave 3), and vmcnt counts in issue order.
+  const bool scale_wave = wave < 3;
+  auto wait_step = [&](int younger) {  // younger: steps issued after the one waited for
+    if (NS == 4 && younger >= 2) {
+      if (scale_wave)
+        asm volatile("s_waitcnt vmcnt(13)" ::: "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+  };
+#pragma unroll
+  for (int a = 0; a < NS - 1; ++a)
+    if (kt_beg + a < kt_end) issue(kt_beg + a);
   for (int kt = kt_beg; kt < nfull; ++kt) {
-    wait_dma_and_sync();  // stage kt&1 holds step kt; everyone is done with the other stage
-    if (kt + 1 < kt_end) issue(kt + 1);
+    wait_step(kt_end - 1 - kt);  // the stage of step kt is complete; everyone is done with the stage of step kt-1
+    if (kt + NS - 1 < kt_end) issue(kt + NS - 1);
     compute(kt, std::false_type{});
   }
   if (tail && kt_beg < kt_end) {
-    wait_dma_and_sync();
+    wait_step(0);
     compute(nk - 1, std::true_type{});
   }
 
@@ -942,12 +963,12 @@ int launch_nvfp4_tiled(const GemmParams &p, hipStream_t st) {
   return ARCQ_OK;
 }
 
-template <int WN, int WM>
+template <int WN, int WM, int NS = 2>
 int launch_mxfp4_tiled(const GemmParams &p, hipStream_t st) {
   constexpr int BN = 64 * WN, BM = 64 * WM;
   const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   const int grid = ((total + 7) / 8) * 8;  // whole groups of 8 so that the XCD split covers every tile
-  hipLaunchKernelGGL((gemm_mxfp4_tiled<WN, WM>), dim3(grid, p.k_slices), dim3(256), 0, st, p);
+  hipLaunchKernelGGL((gemm_mxfp4_tiled<WN, WM, NS>), dim3(grid, p.k_slices), dim3(256), 0, st, p);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }
@@ -1002,7 +1023,7 @@ int launch_tiled_splitk(GemmParams p, int slices, hipStream_t st) {
   p.k_slices = slices;
   p.partial = splitk_workspace();
   if (!p.partial || (size_t)slices * p.M * p.N * sizeof(float) > kSplitWorkspaceBytes) return -1;
-  const int rc = FMT == ARCQ_FMT_MXFP4 ? launch_mxfp4_tiled<2, 1>(p, st) : launch_nvfp4_tiled<2, 1>(p, st);
+  const int rc = FMT == ARCQ_FMT_MXFP4 ? launch_mxfp4_tiled<2, 1, 4>(p, st) : launch_nvfp4_tiled<2, 1>(p, st);
   if (rc != ARCQ_OK) return rc;
   const size_t total4 = ((size_t)p.M * p.N) >> 2;
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<size_t>((total4 + 255) / 256, 1024)), dim3(256), 0, st, p);
@@ -1075,7 +1096,7 @@ static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_
   if (split_env > 1) split = M <= 64 ? split_env : 0;
   else if (split_env == 0 && force < 0 && N <= 8192) {
     if (Kp >= 8192 && M >= 24 && M <= 64) split = 8;
-    else if (Kp < 8192 && N > 4096 && M > 32 && M <= 64) split = 4;
+    else if (Kp < 8192 && N > 4096 && M > (fmt == ARCQ_FMT_MXFP4 ? 16 : 32) && M <= 64) split = 4;
   }
   if (split > 1 && fast_ok && Kp >= 512 && (N & 3) == 0) {
     const int slices = std::min(split, (Kp + 255) / 256 / 2);
@@ -1102,6 +1123,10 @@ static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_
     if (force == 42 || (force < 0 && pick == 42)) return launch_mxfp4_tiled<4, 2>(p, st);
     if (force == 24) return launch_mxfp4_tiled<2, 4>(p, st);
     if (force == 22 || (force < 0 && pick == 22)) return launch_mxfp4_tiled<2, 2>(p, st);
+    // one row of 128x64 tiles (a decode batch): at most one workgroup per CU, whose K steps are short
+    // next to the memory latency -- three steps in flight instead of one (four-stage ring; the same
+    // ring measured no gain for NVFP4, whose steps are long: decoding bounds them)
+    if (force == 214 || (force < 0 && M <= 64)) return launch_mxfp4_tiled<2, 1, 4>(p, st);
     if (force == 21 || force < 0) return launch_mxfp4_tiled<2, 1>(p, st);
   }
   if (fmt == ARCQ_FMT_NVFP4 && force != 0 && tiled_ok) {
