@@ -346,7 +346,7 @@ __device__ __forceinline__ v8i fp4_operand(uint4 q) {
 template <int WN, int WM, int NS = 2>
 __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
   constexpr int BN = 64 * WN, BM = 64 * WM;
-  static_assert(NS == 2 || (NS == 4 && WN == 2 && WM == 1), "the four-stage ring's wait counts are those of the 128x64 tile");
+  static_assert(NS == 2 || (NS == 4 && WN == 2 && WM <= 2), "the four-stage ring's wait counts are those of the 128x64 and 128x128 tiles");
   __shared__ uint4 sW[NS * BN * 8], sX[NS * BM * 8];  // code tiles, NS stages each
   __shared__ uint4 sWs[NS * BN], sXs[NS * BM];        // 16 scale bytes per row (two K steps), NS stages each
   const int tid = threadIdx.x, lane = tid & 63;
@@ -492,13 +492,16 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
   const bool tail = short_last && kt_end == nk;
   const int nfull = tail ? kt_end - 1 : kt_end;
   // NS - 1 steps are on their way while one is computed.  With two stages the wait for a step is a
-  // wait for everything; with four, the two younger steps stay outstanding: this wave issued 6 code
-  // loads for each of them and, for the even one of the two, its share of the scale loads (one
-  // instruction for waves 0..2, none for wave 3), and vmcnt counts in issue order.
-  const bool scale_wave = wave < 3;
+  // wait for everything; with four, the two younger steps stay outstanding: this wave issued
+  // 2*WN + 2*WM code loads for each of them and, for the even one of the two, its share of the scale
+  // loads (128x64 tile: one instruction for waves 0..2, none for wave 3; 128x128: one for every wave),
+  // and vmcnt counts in issue order.
+  const bool scale_wave = WM == 2 || wave < 3;
   auto wait_step = [&](int younger) {  // younger: steps issued after the one waited for
     if (NS == 4 && younger >= 2) {
-      if (scale_wave)
+      if (WM == 2)
+        asm volatile("s_waitcnt vmcnt(17)" ::: "memory");
+      else if (scale_wave)
         asm volatile("s_waitcnt vmcnt(13)" ::: "memory");
       else
         asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
@@ -1093,10 +1096,22 @@ static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_
   // ARCQ_GEMM_SPLITK=<slices> forces it for M <= 64, =1 switches it off.
   static const int split_env = getenv("ARCQ_GEMM_SPLITK") ? atoi(getenv("ARCQ_GEMM_SPLITK")) : 0;
   int split = 0;
-  if (split_env > 1) split = M <= 64 ? split_env : 0;
-  else if (split_env == 0 && force < 0 && N <= 8192) {
-    if (Kp >= 8192 && M >= 24 && M <= 64) split = 8;
-    else if (Kp < 8192 && N > 4096 && M > (fmt == ARCQ_FMT_MXFP4 ? 16 : 32) && M <= 64) split = 4;
+  bool one_round_21 = false;  // 128x64 tiles, no more of them than CUs, K not cut
+  if (split_env > 1) split = M <= 512 ? split_env : 0;
+  else if (split_env == 0 && force < 0 && M <= 64 && N <= 8192) {
+    if (Kp >= 8192 && M >= 24) split = 8;
+    else if (Kp < 8192 && N > 4096 && M > (fmt == ARCQ_FMT_MXFP4 ? 16 : 32)) split = 4;
+  } else if (split_env == 0 && force < 0 && M > 64 && M <= 512) {
+    // Up to a few hundred rows on a narrow layer: the larger tiles leave most CUs without a workgroup,
+    // and a workgroup's time is its number of K steps times the memory latency, whatever M is.  As
+    // many 128x64 tiles x K slices as there are CUs; two slices anyway when K is long.
+    const long tiles21 = (long)((M + 63) / 64) * ((N + 127) / 128);
+    if (tiles21 <= 256) {
+      int sl = Kp >= 8192 ? std::max(2, (int)(256 / tiles21)) : 1;
+      if (fmt == ARCQ_FMT_NVFP4 && Kp < 8192) sl = (int)(256 / tiles21);  // no ring there: slices hide the latency
+      if (sl >= 2) split = std::min(sl, 8);
+      else one_round_21 = true;
+    }
   }
   if (split > 1 && fast_ok && Kp >= 512 && (N & 3) == 0) {
     const int slices = std::min(split, (Kp + 255) / 256 / 2);
@@ -1118,22 +1133,29 @@ static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_
     const long t22 = (long)((M + 127) / 128) * ((N + 127) / 128);
     const double c44 = (double)((t44 + 255) / 256) * 3.08, c42 = (double)((t42 + 255) / 256) * 2.0;
     const double c22 = t22 <= 256 ? 1.33 : (double)((t22 + 511) / 512) * 2.67;
-    const int pick = M <= 128 ? 21 : (M < 512 ? 22 : (c44 < c42 && c44 < c22 ? 44 : (c42 <= c22 ? 42 : 22)));
+    // Problems of one round of workgroups are bounded by the memory latency of their K steps, not by
+    // the matrix cores: the smallest tile that still fits one round (most CUs busy), with three K steps
+    // in flight instead of one (four-stage LDS ring, one workgroup per CU).  The same ring measured
+    // no gain for NVFP4, whose steps are long: decoding bounds them.
+    const long t21 = (long)((M + 63) / 64) * ((N + 127) / 128);
+    const int pick = t21 <= 256 ? 214
+                                : (t22 <= 256 ? 224
+                                              : (M <= 128 ? 21
+                                                          : (M < 512 ? 22
+                                                                     : (c44 < c42 && c44 < c22 ? 44 : (c42 <= c22 ? 42 : 22)))));
     if (force == 44 || (force < 0 && pick == 44)) return launch_mxfp4_tiled<4, 4>(p, st);
     if (force == 42 || (force < 0 && pick == 42)) return launch_mxfp4_tiled<4, 2>(p, st);
     if (force == 24) return launch_mxfp4_tiled<2, 4>(p, st);
+    if (force == 224 || (force < 0 && pick == 224)) return launch_mxfp4_tiled<2, 2, 4>(p, st);
     if (force == 22 || (force < 0 && pick == 22)) return launch_mxfp4_tiled<2, 2>(p, st);
-    // one row of 128x64 tiles (a decode batch): at most one workgroup per CU, whose K steps are short
-    // next to the memory latency -- three steps in flight instead of one (four-stage ring; the same
-    // ring measured no gain for NVFP4, whose steps are long: decoding bounds them)
-    if (force == 214 || (force < 0 && M <= 64)) return launch_mxfp4_tiled<2, 1, 4>(p, st);
+    if (force == 214 || (force < 0 && pick == 214)) return launch_mxfp4_tiled<2, 1, 4>(p, st);
     if (force == 21 || force < 0) return launch_mxfp4_tiled<2, 1>(p, st);
   }
   if (fmt == ARCQ_FMT_NVFP4 && force != 0 && tiled_ok) {
     if (force == 44 || (force < 0 && M > 1024)) return launch_nvfp4_tiled<4, 4>(p, st);
     if (force == 42) return launch_nvfp4_tiled<4, 2>(p, st);
     if (force == 34) return launch_nvfp4_tiled<3, 4>(p, st);
-    if (force == 22 || (force < 0 && M > 128)) return launch_nvfp4_tiled<2, 2>(p, st);
+    if (force == 22 || (force < 0 && M > 128 && !one_round_21)) return launch_nvfp4_tiled<2, 2>(p, st);
     if (force == 21 || force < 0) return launch_nvfp4_tiled<2, 1>(p, st);
   }
   if (fmt == ARCQ_FMT_MXFP4)
