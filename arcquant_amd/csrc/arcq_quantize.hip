@@ -665,19 +665,35 @@ __global__ __launch_bounds__(256) void tensor_scale_kernel(const uint16_t *x, co
   const int cpr = K >> 3;  // 16-byte chunks per row
   const size_t total = (size_t)rows * cpr;
   uint32_t m = 0u;
-  for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < total; c += (size_t)gridDim.x * blockDim.x) {
-    const size_t r = c / cpr, k = (c % cpr) << 3;
-    const uint4 g = *reinterpret_cast<const uint4 *>(x + r * ld + k);
-    uint32_t t[4] = {g.x, g.y, g.z, g.w};
-    if (SWIGLU) {
-      const uint4 u = *reinterpret_cast<const uint4 *>(up + r * ld + k);
-      t[0] = swiglu_pair(g.x, u.x), t[1] = swiglu_pair(g.y, u.y), t[2] = swiglu_pair(g.z, u.z), t[3] = swiglu_pair(g.w, u.w);
+  // four chunks per thread and trip, all loads first: the blocks end in two atomics on the same two
+  // words, which serialise, so a small tensor wants few blocks and still many loads in flight
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t c0 = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c0 < total; c0 += 4 * stride) {
+    uint4 g[4], u[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const size_t c = c0 + j * stride;
+      g[j] = make_uint4(0, 0, 0, 0);
+      u[j] = g[j];
+      if (c < total) {
+        const size_t r = c / cpr, k = (c % cpr) << 3;
+        g[j] = *reinterpret_cast<const uint4 *>(x + r * ld + k);
+        if (SWIGLU) u[j] = *reinterpret_cast<const uint4 *>(up + r * ld + k);
+      }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t lo = (t[i] << 16) & 0x7fffffffu, hi = t[i] & 0x7fff0000u;
-      m = lo > m ? lo : m;
-      m = hi > m ? hi : m;
+    for (int j = 0; j < 4; ++j) {  // an absent chunk is zeros: act_fn(0) * 0 = 0 leaves the maximum alone
+      uint32_t t[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
+      if (SWIGLU) {
+        t[0] = swiglu_pair(g[j].x, u[j].x), t[1] = swiglu_pair(g[j].y, u[j].y);
+        t[2] = swiglu_pair(g[j].z, u[j].z), t[3] = swiglu_pair(g[j].w, u[j].w);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = (t[i] << 16) & 0x7fffffffu, hi = t[i] & 0x7fff0000u;
+        m = lo > m ? lo : m;
+        m = hi > m ? hi : m;
+      }
     }
   }
 #pragma unroll
@@ -689,8 +705,11 @@ __global__ __launch_bounds__(256) void tensor_scale_kernel(const uint16_t *x, co
   __syncthreads();
   if (threadIdx.x != 0) return;
   for (int w = 1; w < 4; ++w) m = wave_max[w] > m ? wave_max[w] : m;
-  const uint32_t old = atomicMax(ws, m);                        // old < 2^31: the next line waits for it
-  const uint32_t arrived = atomicAdd(ws + 1, 1u + (old >> 31));
+  // atomics on one word serialise: a block whose maximum is no larger than what the word already
+  // holds (it only grows, so a value read earlier is a lower bound) has nothing to add
+  uint32_t old = __hip_atomic_load(ws, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (m > old) old = atomicMax(ws, m);
+  const uint32_t arrived = atomicAdd(ws + 1, 1u + (old >> 31));  // old < 2^31: the add waits for the line above
   if (arrived != gridDim.x - 1) return;
   const float amax = u2f(atomicMax(ws, 0u));
   const float scale = amax / divisor;
@@ -973,7 +992,7 @@ int arcq_tensor_scale(const void *x, const void *up, int ld, int M, int K, float
   uint32_t *ws = arcq::tensor_scale_workspace();
   if (!ws) return ARCQ_ERR_LAUNCH;
   const size_t chunks = (size_t)M * (K >> 3);
-  int grid = (int)((chunks + 255) / 256 < 1024 ? (chunks + 255) / 256 : 1024);
+  int grid = (int)((chunks + 1023) / 1024 < 1024 ? (chunks + 1023) / 1024 : 1024);  // four chunks per thread
   if (grid < 1) grid = 1;  // M == 0: one block writes the scale of an empty tensor, 1
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (up)
