@@ -92,9 +92,13 @@ def test_identity_weights_recover_activations(agemm, oracle, fmt):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-@pytest.mark.parametrize("M,N,K,S", [(512, 4096, 4096, 256), (2048, 6144, 4096, 256), (256, 4096, 14336, 256)])
+@pytest.mark.parametrize("M,N,K,S", [(512, 4096, 4096, 256), (2048, 6144, 4096, 256), (256, 4096, 14336, 256),
+                                     (512, 6144, 1024, 128), (448, 6200, 768, 256), (128, 28672, 1024, 256),
+                                     (100, 4096, 4096, 256), (384, 4100, 8192, 128)])
 def test_matmul_llama_shapes_vs_torch_fp32(agemm, fmt, M, N, K, S):
-    """Benchmark shapes: compare with torch's fp32 matmul of the dequantized operands on the GPU."""
+    """Benchmark shapes, and shapes of one round of workgroups (at most 256 tiles of 128x64 or 128x128, also
+    ragged and with K' % 256 == 128, and K cut into slices for a few hundred rows): compare with torch's
+    fp32 matmul of the dequantized operands on the GPU."""
     (x, w, idx, gx, gw), (a, sfa, b, sfb) = quantized_pair(agemm, M, N, K, S, fmt, seed=3)
     print(f"matmul {fmt} M={M} N={N} K={K} S={S}", flush=True)
     y = agemm.matmul(a, b, sfa, sfb, gx * gw)
@@ -150,6 +154,8 @@ def test_matmul_decode_batches(agemm, fmt, M, N, K, S):
     (33, 28672, 1024, 128),    # tiled 128x64
     (40, 8324, 1024, 256),     # tiled 128x64, ragged last workgroup
     (300, 1000, 2048, 128),    # tiled, ragged M and N: transposed epilogue and the per-element one
+    (512, 6144, 1024, 128),    # one round of 128x128 tiles
+    (200, 4096, 8448, 256),    # a few hundred rows, long K: slices
     (1100, 1024, 1024, 0),     # 256x256 tiles (MXFP4 cost model may take smaller ones) with a ragged M
     (130, 384, 448, 64),       # K' % 128 != 0: direct kernels
     (5, 202, 384, 0),          # N % 4 != 0: scalar stores
