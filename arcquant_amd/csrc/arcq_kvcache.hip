@@ -430,6 +430,16 @@ __device__ __forceinline__ v8h k_operand(uint32_t x) {
 // MFMAs), so the kernel lives on waves per SIMD, and batch x KV heads workgroups of four waves give
 // only two.
 constexpr int kDecodeWaves = 8;
+// Chunks travel global -> LDS without passing through registers (global_load_lds), four per wave in
+// flight, each wave into its own slots: codes of K (1 KB), codes of V (1 KB), the 32 parameter words.
+constexpr int kDecodeStages = 4;
+constexpr int kDecodeSlotBytes = 1024 + 1024 + 128;
+__device__ __forceinline__ void kv_lds_dma16(const void *g, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_wave_base), "v"(g) : "memory");
+}
+__device__ __forceinline__ void kv_lds_dma4(const void *g, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(lds_wave_base), "v"(g) : "memory");
+}
 // With few sequences the (sequence, KV head) grid leaves CUs idle: gridDim.z > 1 cuts every sequence's
 // chunks into that many ranges, one workgroup each, which write (maximum, denominator, numerator[128])
 // per head to `partial` instead of the output; kv_decode_merge_kernel combines them.
@@ -438,10 +448,13 @@ template <bool BF16, int G>
 __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(uint16_t *o, const uint16_t *q, KvLayout c,
                                                                               int num_qo_heads, float sm_scale_log2,
                                                                               float *partial) {
-  __shared__ float part_o[kDecodeWaves][G][kHeadDim];
-  __shared__ float part_s[kDecodeWaves][G][4];  // m, l, D (1024 * sum of P), Z (sum of p * zero)
+  // the waves' partial results meet, after the loop, in the memory of the slots
+  __shared__ uint4 slots[kDecodeWaves * kDecodeStages * kDecodeSlotBytes / 16];
+  static_assert(sizeof(float) * kDecodeWaves * G * (kHeadDim + 4) <= sizeof(slots), "the merge area lies inside the slots");
+  float(*part_o)[G][kHeadDim] = reinterpret_cast<float(*)[G][kHeadDim]>(slots);
+  float(*part_s)[G][4] = reinterpret_cast<float(*)[G][4]>(reinterpret_cast<float *>(slots) + kDecodeWaves * G * kHeadDim);  // m, l, D (1024 * sum of P), Z (sum of p * zero)
   const int b = blockIdx.x, h = blockIdx.y;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
   const int p0 = c.indptr[b], np = c.indptr[b + 1] - p0;
   const int len = np > 0 ? (np - 1) * c.page_size + c.last_page_offset[b] : 0;
@@ -483,18 +496,57 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(ui
 
   const int nchunks = (len + 15) >> 4;
   const int ch_beg = (int)((long)nchunks * blockIdx.z / gridDim.z), ch_end = (int)((long)nchunks * (blockIdx.z + 1) / gridDim.z);
-  for (int ch = ch_beg + wave; ch < ch_end; ch += kDecodeWaves) {
-    const int t0 = ch << 4;
-    const int page = c.indices[p0 + t0 / c.page_size], slot0 = t0 % c.page_size;
+  // this wave's chunks: ch_beg + wave + kDecodeWaves * k, k = 0 .. n_mine-1
+  const int n_mine = ch_end > ch_beg + wave ? (ch_end - ch_beg - wave + kDecodeWaves - 1) / kDecodeWaves : 0;
+  const uint32_t slot_base = (uint32_t)reinterpret_cast<uintptr_t>(slots) + wave * (kDecodeStages * kDecodeSlotBytes);
+  // The pages of this wave's chunks, 64 at a time, one per lane: inside the loop a page is a readlane,
+  // not a load (a load there would be waited for with vmcnt(0), draining the chunks in flight; that
+  // happens once per 64 chunks).
+  int pages = 0;
+  auto load_pages = [&](int k0) {
+    const int kk = k0 + lane;
+    pages = kk < n_mine ? c.indices[p0 + ((ch_beg + wave + kDecodeWaves * kk) << 4) / c.page_size] : 0;
+  };
+  auto page_of = [&](int k) { return __builtin_amdgcn_readlane(pages, k & 63); };  // k in the block last loaded
+  // V travels so that the dword a lane needs of token 4g+i sits at 256 i + 4 lane of the slot: the lane
+  // that fetches 16 bytes into position L of the slot takes token 4 ((L >> 2) & 3) + (L >> 4), piece L & 3
+  const int v_tok = 4 * ((lane >> 2) & 3) + (lane >> 4), v_piece = lane & 3;
+  auto issue = [&](int k, int page) {  // three instructions per chunk and wave: vmcnt counts on it
+    if (k >= n_mine) return;  // wave-uniform
+    const int t0 = (ch_beg + wave + kDecodeWaves * k) << 4, slot0 = t0 % c.page_size;
     const size_t krow0 = kv_row(c, page, 0, h, slot0), vrow0 = kv_row(c, page, 1, h, slot0);
-    // K: this lane's token r16, bytes 16g .. 16g+15
-    const uint4 kq = reinterpret_cast<const uint4 *>(c.data + (krow0 + r16) * kRowBytes)[g];
-    // V: dword r16 (dims 8 r16 ..) of tokens 4g .. 4g+3
+    const uint32_t dst = slot_base + (k % kDecodeStages) * kDecodeSlotBytes;
+    kv_lds_dma16(c.data + (krow0 + r16) * kRowBytes + 16 * g, dst);                   // K: token r16, bytes 16g .. 16g+15
+    kv_lds_dma16(c.data + (vrow0 + v_tok) * kRowBytes + 16 * v_piece, dst + 1024);
+    if (lane < 32) kv_lds_dma4(c.param + (lane < 16 ? krow0 + lane : vrow0 + lane - 16), dst + 2048);
+  };
+  load_pages(0);
+  issue(0, page_of(0));
+  issue(1, page_of(1));
+  issue(2, page_of(2));
+  for (int k = 0; k < n_mine; ++k) {
+    const int ch = ch_beg + wave + kDecodeWaves * k;
+    const int t0 = ch << 4;
+    if (((k + 3) & 63) == 0) load_pages(k + 3);
+    issue(k + 3, page_of(k + 3));
+    const int younger = n_mine - 1 - k;  // chunks asked for after this one
+    if (younger >= 3)
+      asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    else if (younger == 2)
+      asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else if (younger == 1)
+      asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const uint8_t *slot = reinterpret_cast<const uint8_t *>(slots) + wave * (kDecodeStages * kDecodeSlotBytes) +
+                          (k % kDecodeStages) * kDecodeSlotBytes;
+    const uint4 kq = reinterpret_cast<const uint4 *>(slot)[lane];
     uint32_t vd[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) vd[i] = reinterpret_cast<const uint32_t *>(c.data + (vrow0 + 4 * g + i) * kRowBytes)[r16];
-    const uint4 kpar = *reinterpret_cast<const uint4 *>(c.param + krow0 + 4 * g);
-    const uint4 vpar = *reinterpret_cast<const uint4 *>(c.param + vrow0 + 4 * g);
+    for (int i = 0; i < 4; ++i) vd[i] = reinterpret_cast<const uint32_t *>(slot + 1024 + 256 * i)[lane];
+    const uint4 kpar = reinterpret_cast<const uint4 *>(slot + 2048)[g];
+    const uint4 vpar = reinterpret_cast<const uint4 *>(slot + 2048 + 64)[g];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot is read before a later request may overwrite it
 
     v4f sacc = {0.f, 0.f, 0.f, 0.f};
     sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.x), qop[0], sacc, 0, 0, 0);
@@ -564,6 +616,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(ui
   d_run += __shfl_xor(d_run, 32);
   z_run += __shfl_xor(z_run, 16);
   z_run += __shfl_xor(z_run, 32);
+  __syncthreads();  // every wave is done with its slots
   if (g == 0) {
     if (r16 < G) {
       part_s[wave][r16][0] = m_run;

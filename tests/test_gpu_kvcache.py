@@ -238,6 +238,34 @@ def test_decode_attention_many_sequences(kvc, ref):
     assert float(o[7].abs().sum()) == 0.0
 
 
+def test_decode_attention_long_sequence_whole(kvc, ref):
+    """256 (sequence, KV head) pairs, so every sequence is taken whole by one workgroup, and one of them
+    long enough (8200 tokens, more than 64 chunks per wave) that the kernel fetches its page numbers in
+    more than one block while chunks are in flight."""
+    batch, q_heads, kv_heads, page_size, dtype = 64, 8, 4, 16, torch.bfloat16
+    g = torch.Generator().manual_seed(29)
+    lengths = [int(n) for n in torch.randint(1, 60, (batch,), generator=g)]
+    lengths[3] = 8200
+    total = sum(lengths)
+    k = torch.randn(total, kv_heads, 128, generator=g).to(dtype)
+    v = torch.randn(total, kv_heads, 128, generator=g).to(dtype)
+    q = torch.randn(batch, q_heads, 128, generator=g).to(dtype)
+    indptr, indices, last, maxc = make_table(lengths, page_size, batch)
+    pages = torch.zeros(maxc * batch, 1, 2, kv_heads, page_size, 64, dtype=torch.uint8, device="cuda")
+    params = torch.full((maxc * batch, 1, 2, kv_heads, page_size, 2), float("nan"), dtype=dtype, device="cuda")
+    offs = [0]
+    for n in lengths:
+        offs.append(offs[-1] + n)
+    print("kv decode, 64 sequences x 4 KV heads, one of 8200 tokens", flush=True)
+    kvc.quantize_append(pages, params, indptr.cuda(), indices.cuda(), last.cuda(), k.cuda(), v.cuda(), 0,
+                        seqlen_indptr=torch.tensor(offs, dtype=torch.int32).cuda(), max_new_tokens=max(lengths))
+    o = torch.full_like(q, 7.0).cuda()
+    kvc.batch_decode_i4(o, q.cuda(), pages, params, indptr.cuda(), indices.cuda(), last.cuda(), 0)
+    want = ref.decode_attention(q, pages.cpu(), params.cpu(), indptr, indices, last, 0)
+    assert rel_fro(o, want) < 5e-3
+    assert rel_fro(o[3], want[3]) < 5e-3
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_rope_rows_match_torch(kvc, dtype):
     """The one-pass rotary embedding of a prompt against torch's q * cos + rotate_half(q) * sin on the
