@@ -429,6 +429,18 @@ __device__ __forceinline__ v8h k_operand(uint32_t x) {
 // dependent steps (loads, four MFMAs on one accumulator, cross-lane maxima, exponentials, eight more
 // MFMAs), so the kernel lives on waves per SIMD, and batch x KV heads workgroups of four waves give
 // only two.
+// maximum over the four lanes L, L^16, L^32, L^48 in every one of them, on the VALU: the lane-swap
+// instructions exchange rows (of 16 lanes) and halves between two registers; with both registers
+// holding m, the two results hold a lane's own value and its partner's
+__device__ __forceinline__ float max_over_lane_groups(float m) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, m);
+  const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  const float m16 = fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+  const uint32_t c = __builtin_bit_cast(uint32_t, m16);
+  const auto q = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+  return fmaxf(__builtin_bit_cast(float, q[0]), __builtin_bit_cast(float, q[1]));
+}
+
 constexpr int kDecodeWaves = 8;
 // Chunks travel global -> LDS without passing through registers (global_load_lds), four per wave in
 // flight, each wave into its own slots: codes of K (1 KB), codes of V (1 KB), the 32 parameter words.
@@ -555,22 +567,23 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(ui
     sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.w), qop[3], sacc, 0, 0, 0);
 
     const uint32_t kp[4] = {kpar.x, kpar.y, kpar.z, kpar.w}, vp[4] = {vpar.x, vpar.y, vpar.z, vpar.w};
+    const bool whole = t0 + 16 <= len;  // wave-uniform: only a sequence's last chunk has rows past the end
     float sc[4], mx = m_run;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const float ks = from_bits<BF16>(kp[v]), kz = from_bits<BF16>(kp[v] >> 16);
-      sc[v] = (t0 + 4 * g + v < len) ? (ks * (sacc[v] - qoff) - kz * qsum) * sm_scale_log2 : kNegBig;
+      sc[v] = (ks * (sacc[v] - qoff) - kz * qsum) * sm_scale_log2;
+      if (!whole && !(t0 + 4 * g + v < len)) sc[v] = kNegBig;
       mx = fmaxf(mx, sc[v]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    mx = max_over_lane_groups(mx);
     const float corr = __builtin_amdgcn_exp2f(m_run - mx);
     m_run = mx;
     v4h pa;
     float psum = 0.0f, pasum = 0.0f, pz = 0.0f;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const bool valid = t0 + 4 * g + v < len;           // rows past the end may hold anything
+      const bool valid = whole || t0 + 4 * g + v < len;  // rows past the end may hold anything
       const float pv = __builtin_amdgcn_exp2f(sc[v] - mx);
       const float vs = valid ? from_bits<BF16>(vp[v]) : 0.0f, vz = valid ? from_bits<BF16>(vp[v] >> 16) : 0.0f;
       psum += pv;
