@@ -20,6 +20,7 @@
 
 #include <algorithm>
 #include <mutex>
+#include <type_traits>
 
 #include "../../include/arcq.h"
 #include "arcq_internal.h"
@@ -403,6 +404,7 @@ __global__ __launch_bounds__(256) void kv_decode_i4_kernel(uint16_t *o, const ui
 // V operand of a lane is one dword (8 dims) of each of its 4 tokens, output column j of MFMA j being
 // dim 8 * (lane % 16) + j.
 // ---------------------------------------------------------------------------------------------
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -415,13 +417,19 @@ typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 // elements that meet a 16 n divided by 16, and the 1024 terms are subtracted from the scores as one
 // number per head (1024 * sum of q over the low-nibble dims + 64 * sum over the high-nibble dims).
 constexpr int kDimOfElem[8] = {0, 4, 1, 5, 2, 6, 3, 7};
-__device__ __forceinline__ v8h k_operand(uint32_t x) {
+// The three constants (0x64006400 = fp16 1024 twice, and the two nibble masks) are held in registers
+// the compiler knows nothing about: this chip's three-operand encoding takes no literal, so with
+// literals (x & mask) | 0x64006400 is two instructions, with registers it is one v_and_or_b32.
+struct NibbleConsts {
+  uint32_t one_k, lo, hi;
+};
+__device__ __forceinline__ v8h k_operand(uint32_t x, const NibbleConsts &k) {
   v4u d;
   const uint32_t y = x >> 8;
-  d[0] = (x & 0x000f000fu) | 0x64006400u;
-  d[1] = (x & 0x00f000f0u) | 0x64006400u;
-  d[2] = (y & 0x000f000fu) | 0x64006400u;
-  d[3] = (y & 0x00f000f0u) | 0x64006400u;
+  d[0] = (x & k.lo) | k.one_k;
+  d[1] = (x & k.hi) | k.one_k;
+  d[2] = (y & k.lo) | k.one_k;
+  d[3] = (y & k.hi) | k.one_k;
   return __builtin_bit_cast(v8h, d);
 }
 
@@ -501,6 +509,8 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(ui
     qoff += __shfl_xor(qoff, 32);
   }
 
+  NibbleConsts nib = {0x64006400u, 0x000f000fu, 0x00f000f0u};
+  asm volatile("" : "+s"(nib.one_k), "+v"(nib.lo), "+v"(nib.hi));
   float m_run = kNegBig, l_run = 0.0f, d_run = 0.0f, z_run = 0.0f;
   v4f oacc[8];
 #pragma unroll
@@ -561,36 +571,51 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(ui
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot is read before a later request may overwrite it
 
     v4f sacc = {0.f, 0.f, 0.f, 0.f};
-    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.x), qop[0], sacc, 0, 0, 0);
-    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.y), qop[1], sacc, 0, 0, 0);
-    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.z), qop[2], sacc, 0, 0, 0);
-    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.w), qop[3], sacc, 0, 0, 0);
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.x, nib), qop[0], sacc, 0, 0, 0);
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.y, nib), qop[1], sacc, 0, 0, 0);
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.z, nib), qop[2], sacc, 0, 0, 0);
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand(kq.w, nib), qop[3], sacc, 0, 0, 0);
 
     const uint32_t kp[4] = {kpar.x, kpar.y, kpar.z, kpar.w}, vp[4] = {vpar.x, vpar.y, vpar.z, vpar.w};
-    const bool whole = t0 + 16 <= len;  // wave-uniform: only a sequence's last chunk has rows past the end
-    float sc[4], mx = m_run;
+    // scores -> running maximum -> P (times the V scales, as fp16) and this chunk's sums.  Only a
+    // sequence's last chunk has rows past the end (they may hold anything): every other chunk takes
+    // the variant without the row masks (the choice is wave-uniform).
+    v2h p01, p23;
+    float corr, psum = 0.0f, pasum, pz = 0.0f;
+    auto scores_to_p = [&](auto whole_c) {
+      constexpr bool WHOLE = decltype(whole_c)::value;
+      float sc[4], mx = m_run;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const float ks = from_bits<BF16>(kp[v]), kz = from_bits<BF16>(kp[v] >> 16);
-      sc[v] = (ks * (sacc[v] - qoff) - kz * qsum) * sm_scale_log2;
-      if (!whole && !(t0 + 4 * g + v < len)) sc[v] = kNegBig;
-      mx = fmaxf(mx, sc[v]);
-    }
-    mx = max_over_lane_groups(mx);
-    const float corr = __builtin_amdgcn_exp2f(m_run - mx);
-    m_run = mx;
-    v4h pa;
-    float psum = 0.0f, pasum = 0.0f, pz = 0.0f;
+      for (int v = 0; v < 4; ++v) {
+        const float ks = from_bits<BF16>(kp[v]), kz = from_bits<BF16>(kp[v] >> 16);
+        sc[v] = (ks * (sacc[v] - qoff) - kz * qsum) * sm_scale_log2;
+        if (!WHOLE && !(t0 + 4 * g + v < len)) sc[v] = kNegBig;
+        mx = fmaxf(mx, sc[v]);
+      }
+      mx = max_over_lane_groups(mx);
+      corr = __builtin_amdgcn_exp2f(m_run - mx);
+      m_run = mx;
+      float pr[4];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const bool valid = whole || t0 + 4 * g + v < len;  // rows past the end may hold anything
-      const float pv = __builtin_amdgcn_exp2f(sc[v] - mx);
-      const float vs = valid ? from_bits<BF16>(vp[v]) : 0.0f, vz = valid ? from_bits<BF16>(vp[v] >> 16) : 0.0f;
-      psum += pv;
-      pz = __builtin_fmaf(pv, vz, pz);
-      pa[v] = (_Float16)(pv * vs);
-      pasum += (float)pa[v];
-    }
+      for (int v = 0; v < 4; ++v) {
+        const bool valid = WHOLE || t0 + 4 * g + v < len;
+        const float pv = __builtin_amdgcn_exp2f(sc[v] - mx);
+        const float vs = valid ? from_bits<BF16>(vp[v]) : 0.0f, vz = valid ? from_bits<BF16>(vp[v] >> 16) : 0.0f;
+        psum += pv;
+        pz = __builtin_fmaf(pv, vz, pz);
+        pr[v] = pv * vs;
+      }
+      p01 = v2h{(_Float16)pr[0], (_Float16)pr[1]};
+      p23 = v2h{(_Float16)pr[2], (_Float16)pr[3]};
+    };
+    if (t0 + 16 <= len)
+      scores_to_p(std::true_type{});
+    else
+      scores_to_p(std::false_type{});
+    // the sum of the four fp16 values as the second product sees them
+    const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
+    pasum = __builtin_amdgcn_fdot2(p01, ones, __builtin_amdgcn_fdot2(p23, ones, 0.0f, false), false);
+    const v4h pa = {p01[0], p01[1], p23[0], p23[1]};
     l_run = l_run * corr + psum;
     d_run = d_run * corr + 1024.0f * pasum;
     z_run = z_run * corr + pz;
@@ -610,10 +635,10 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void kv_decode_i4_mfma_kernel(ui
     const uint32_t t01 = __builtin_amdgcn_perm(vd[1], vd[0], 0x0c040c00u + 0x00010001u * (BB));                 \
     const uint32_t t23 = __builtin_amdgcn_perm(vd[3], vd[2], 0x0c040c00u + 0x00010001u * (BB));                 \
     v2u lo, hi;                                                                                                 \
-    lo[0] = (t01 & 0x000f000fu) | 0x64006400u;                                                                  \
-    lo[1] = (t23 & 0x000f000fu) | 0x64006400u;                                                                  \
-    hi[0] = (t01 & 0x00f000f0u) | 0x64006400u;                                                                  \
-    hi[1] = (t23 & 0x00f000f0u) | 0x64006400u;                                                                  \
+    lo[0] = (t01 & nib.lo) | nib.one_k;                                                                         \
+    lo[1] = (t23 & nib.lo) | nib.one_k;                                                                         \
+    hi[0] = (t01 & nib.hi) | nib.one_k;                                                                         \
+    hi[1] = (t23 & nib.hi) | nib.one_k;                                                                         \
     oacc[2 * (BB)] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa, __builtin_bit_cast(v4h, lo), oacc[2 * (BB)], 0, 0, 0);      \
     oacc[2 * (BB) + 1] =                                                                                        \
         __builtin_amdgcn_mfma_f32_16x16x16f16(pa, __builtin_bit_cast(v4h, hi), oacc[2 * (BB) + 1], 0, 0, 0);    \
