@@ -41,6 +41,8 @@ def lib() -> ctypes.CDLL:
     L.arcq_status_string.argtypes = [i]
     L.arcq_status_string.restype = ctypes.c_char_p
     L.arcq_last_hip_error.restype = i
+    L.arcq_prepare_stream.argtypes = [vp]
+    L.arcq_prepare_stream.restype = i
     L.arcq_group_size.argtypes = [i]
     L.arcq_group_size.restype = i
     L.arcq_codes_bytes.argtypes = [i, i, i]
@@ -61,6 +63,12 @@ def lib() -> ctypes.CDLL:
     L.arcq_kv_decode_i4.argtypes = [vp, vp, i, i, i, vp, vp, vp, vp, vp, i, i, i, i, i, f, vp]
     L.arcq_matmul.argtypes = [vp, vp, vp, vp, i, i, i, i, f, vp, vp, vp, vp]
     L.arcq_matmul_add.argtypes = [vp, vp, vp, vp, i, i, i, i, f, vp, vp, vp, vp, vp]
+    if hasattr(L, "arcq_matmul_noalloc"):
+        L.arcq_matmul_noalloc.argtypes = L.arcq_matmul.argtypes
+        L.arcq_matmul_noalloc.restype = i
+        L.arcq_matmul_noalloc_limit.restype = sz
+        L.arcq_matmul_scratch_bytes.argtypes = [i, i, i, i]
+        L.arcq_matmul_scratch_bytes.restype = sz
     L.arcq_check_index.argtypes = [vp, i, vp]
     L.arcq_dequantize.argtypes = [vp, vp, i, i, i, vp, vp]
     L.arcq_stream_probe.argtypes = [vp, vp, sz, sz, vp]

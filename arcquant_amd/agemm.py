@@ -30,8 +30,8 @@ import torch
 from . import _lib
 from ._lib import FORMATS, ArcqError  # noqa: F401
 
-__all__ = ["matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "swiglu_quantize_x", "dequantize",
-           "check_index",
+__all__ = ["matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "init_kv_i4", "append_kv_i4",
+           "batch_decode_i4", "swiglu_quantize_x", "tensor_scale", "prepare_stream", "dequantize", "check_index",
            "unpack_codes", "scale_values"]
 
 
@@ -241,6 +241,20 @@ def matmul(A, B, SFA, SFB, scale, *, fmt=None, residual=None):
     _lib.check(rc, "arcq_matmul")
     del ka, kb
     return C
+
+
+def prepare_stream(device=None) -> None:
+    """Allocate the library's scratch buffers for torch's current stream on `device` (arcq_prepare_stream).
+    Needed once per stream before a capture on it: a captured call cannot allocate."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    probe = torch.empty(0, device=dev)
+    with _on_device(probe):
+        _lib.check(_lib.lib().arcq_prepare_stream(_stream(probe)), "arcq_prepare_stream")
+
+
+# The three INT4 KV-cache operators of the reference's module (kernels/src/bindings.cpp:576-578), so that a
+# caller written against `agemm` (model/kv_cache.py:49-80) finds them here; same keyword arguments.
+from .kv_cache import append_kv_i4, batch_decode_i4, init_kv_i4  # noqa: E402,F401
 
 
 # ------------------------------------------------------------------------------------------

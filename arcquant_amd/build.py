@@ -1,6 +1,6 @@
-"""Builds libarcq_hip.so (gfx950) and libarcq_hostmath.so in-tree with hipcc / g++.
+"""Builds libarcq_hip.so (gfx950) in-tree with hipcc.
 
-    python -m arcquant_amd.build            # build both
+    python -m arcquant_amd.build            # build if stale
     python -m arcquant_amd.build --force    # rebuild even if up to date
 
 hipcc cross-compiles for gfx950 without a GPU present.  The built libraries live next to the
@@ -17,7 +17,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 HIP_SOURCES = ["arcq_common.hip", "arcq_quantize.hip", "arcq_gemm.hip", "arcq_kvcache.hip"]
 HIP_LIB = os.path.join(CSRC, "libarcq_hip.so")
-HOST_LIB = os.path.join(CSRC, "libarcq_hostmath.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -55,19 +54,8 @@ def build_hip(force: bool = False, verbose: bool = False) -> str:
     return HIP_LIB
 
 
-def build_hostmath(force: bool = False, verbose: bool = False) -> str:
-    src = os.path.join(CSRC, "host_math.cpp")
-    if force or _stale(HOST_LIB, [src, os.path.join(CSRC, "arcq_math.h")]):
-        cmd = ["g++", "-O2", "-std=c++20", "-fPIC", "-shared", "-fopenmp", "-msse2", "-mfpmath=sse", "-mfma",
-               "-ffp-contract=off", "-o", HOST_LIB, src]
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        subprocess.check_call(cmd)
-    return HOST_LIB
-
-
 def build_all(force: bool = False, verbose: bool = False):
-    return build_hip(force, verbose), build_hostmath(force, verbose)
+    return (build_hip(force, verbose),)
 
 
 if __name__ == "__main__":

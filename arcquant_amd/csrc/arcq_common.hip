@@ -1,22 +1,85 @@
-// arcq_common.hip -- status strings, version, last-error bookkeeping of libarcq_hip.so.
+// arcq_common.hip -- status strings, version, last-error bookkeeping, per-stream scratch memory and
+// the tuning overrides of libarcq_hip.so.
 #include <hip/hip_runtime.h>
+#include <stdlib.h>
+
+#include <mutex>
+#include <vector>
 
 #include "arcq_internal.h"
 
 namespace arcq {
 namespace {
 thread_local int g_last_hip_error = 0;
-}
+
+struct WorkspaceEntry {
+  int device;
+  hipStream_t stream;
+  void *ptr[kWsKinds];
+};
+std::mutex g_ws_mutex;
+std::vector<WorkspaceEntry> g_ws;  // a few entries: one per (device, stream) that ever needed scratch
+}  // namespace
 
 int note_hip_error(hipError_t e) {
   g_last_hip_error = static_cast<int>(e);
   return ARCQ_ERR_LAUNCH;
 }
+
+void *stream_workspace(int kind, hipStream_t stream, int *status) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    *status = note_hip_error(e);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  WorkspaceEntry *ent = nullptr;
+  for (auto &w : g_ws)
+    if (w.device == dev && w.stream == stream) ent = &w;
+  if (ent && ent->ptr[kind]) return ent->ptr[kind];
+  // nothing yet: allocate, unless the stream is being captured (hipMalloc there would end the capture)
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
+  if (cap != hipStreamCaptureStatusNone) {
+    *status = ARCQ_ERR_WORKSPACE;
+    return nullptr;
+  }
+  void *p = nullptr;
+  e = hipMalloc(&p, kWorkspaceBytes[kind]);
+  if (e == hipSuccess && kind == kWsTensorScale) {
+    e = hipMemsetAsync(p, 0, kWorkspaceBytes[kind], stream);  // ordered in front of the first kernel that uses it
+    if (e != hipSuccess) (void)hipFree(p);
+  }
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    *status = note_hip_error(e);
+    return nullptr;
+  }
+  if (!ent) {
+    g_ws.push_back(WorkspaceEntry{dev, stream, {nullptr, nullptr, nullptr}});
+    ent = &g_ws.back();
+  }
+  ent->ptr[kind] = p;
+  return p;
+}
+
+const Tuning &tuning() {
+  static const Tuning t = [] {
+    Tuning v;
+    if (const char *e = getenv("ARCQ_GEMM_KERNEL")) v.gemm_kernel = atoi(e);
+    if (const char *e = getenv("ARCQ_GEMM_SPLITK")) v.gemm_splitk = atoi(e);
+    if (const char *e = getenv("ARCQ_QUANT_GRID")) v.quant_grid = atoi(e);
+    if (const char *e = getenv("ARCQ_KV_DECODE_SPLITS")) v.kv_decode_splits = atoi(e);
+    return v;
+  }();
+  return t;
+}
 }  // namespace arcq
 
 extern "C" {
 
-int arcq_version(void) { return 100; }  // 0.1.0
+int arcq_version(void) { return 200; }  // 0.2.0
 
 const char *arcq_status_string(int status) {
   switch (status) {
@@ -28,10 +91,22 @@ const char *arcq_status_string(int status) {
     case ARCQ_ERR_ALIGN: return "a pointer is not 16-byte aligned";
     case ARCQ_ERR_LAUNCH: return "HIP launch failed";
     case ARCQ_ERR_INDEX: return "reorder_index is not a permutation of 0..K-1";
+    case ARCQ_ERR_WORKSPACE: return "scratch memory unavailable: the stream is being captured and has none yet (call "
+                                    "arcq_prepare_stream before the capture), or the problem exceeds the fixed scratch "
+                                    "of a non-allocating entry point";
     default: return "unknown status";
   }
 }
 
 int arcq_last_hip_error(void) { return arcq::g_last_hip_error; }
+
+int arcq_prepare_stream(void *stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  for (int kind = 0; kind < arcq::kWsKinds; ++kind) {
+    int status = ARCQ_OK;
+    if (!arcq::stream_workspace(kind, st, &status)) return status;
+  }
+  return ARCQ_OK;
+}
 
 }  // extern "C"

@@ -239,11 +239,15 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_direct(GemmParams p) {
 // MFMAs, so its four E8M0 bytes are one dword of the row-major scale array and the byte is
 // picked by the instruction's op_sel.
 // ---------------------------------------------------------------------------------------------
+// These write M0.  The compiler reserves M0 and refuses it on a clobber list ("may lead to undefined
+// behaviour"), so the contract is kept by hand: the kernels that use these helpers contain nothing for
+// which the compiler would set or read M0 itself (no LDS-direct builtins, no indirect register
+// indexing, no s_sendmsg), and every helper sets M0 before its load.
 __device__ __forceinline__ void lds_dma16(const void *g, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                :
                : "s"(lds_wave_base), "v"(g)
-               : "memory");  // M0 is written; nothing else in these kernels reads it
+               : "memory");
 }
 
 __device__ __forceinline__ void lds_dma4(const void *g, uint32_t lds_wave_base) {
@@ -948,11 +952,8 @@ int launch_skinny(const GemmParams &p, hipStream_t st) {
 
 template <int FMT>
 int launch_skinny_for(const GemmParams &p, hipStream_t st) {
-  // two 16-row weight tiles per wave (halving the activation reads) measured no better: experiments only
-  static const int at_env = getenv("ARCQ_GEMM_SKINNY_AT") ? atoi(getenv("ARCQ_GEMM_SKINNY_AT")) : 0;
-  const bool at2 = FMT == ARCQ_FMT_MXFP4 && at_env == 2;
-  if (p.M <= 16) return at2 ? launch_skinny<FMT, 1, 2>(p, st) : launch_skinny<FMT, 1, 1>(p, st);
-  if (p.M <= 32) return at2 ? launch_skinny<FMT, 2, 2>(p, st) : launch_skinny<FMT, 2, 1>(p, st);
+  if (p.M <= 16) return launch_skinny<FMT, 1, 1>(p, st);
+  if (p.M <= 32) return launch_skinny<FMT, 2, 1>(p, st);
   return launch_skinny<FMT, 4, 1>(p, st);
 }
 
@@ -998,93 +999,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p) {
   }
 }
 
-// Workspace of the partial tiles: one per device, allocated on the first call that needs it and kept
-// until the process ends (a captured graph may hold its address).  Calls that overlap in time on one
-// device would share it; launches are stream-ordered as everywhere else in this library.
-constexpr size_t kSplitWorkspaceBytes = 32u << 20;
-constexpr int kSplitMaxDevices = 16;
+// Which kernel runs a problem, decided on the host from the shape alone (so that every entry point
+// that shares this plan computes the same bits).  kernel: 0 = direct, 1 = skinny, <WN><WM> = tiled
+// (214 / 224: MXFP4 with the four-stage ring); slices > 1: split-K over 128x64 tiles, which needs
+// slices * M * N fp32 words of scratch.
+struct GemmPlan {
+  int kernel = 0;
+  int slices = 1;
+  size_t scratch_bytes() const { return slices > 1 ? scratch : 0; }
+  size_t scratch = 0;
+};
 
-inline float *splitk_workspace() {
-  static std::mutex mu;
-  static float *ws[kSplitMaxDevices];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kSplitMaxDevices) return nullptr;
-  std::lock_guard<std::mutex> lock(mu);
-  if (!ws[dev]) {
-    float *w = nullptr;
-    if (hipMalloc(&w, kSplitWorkspaceBytes) != hipSuccess) {
-      (void)hipGetLastError();  // e.g. under stream capture before any eager call: the caller runs without split-K
-      return nullptr;
-    }
-    ws[dev] = w;
-  }
-  return ws[dev];
-}
+// the largest scratch the plan ever asks for (the stream workspaces are this big)
+constexpr size_t kSplitMaxBytes = kWorkspaceBytes[kWsSplitK];
 
-template <int FMT>
-int launch_tiled_splitk(GemmParams p, int slices, hipStream_t st) {
-  p.k_slices = slices;
-  p.partial = splitk_workspace();
-  if (!p.partial || (size_t)slices * p.M * p.N * sizeof(float) > kSplitWorkspaceBytes) return -1;
-  const int rc = FMT == ARCQ_FMT_MXFP4 ? launch_mxfp4_tiled<2, 1, 4>(p, st) : launch_nvfp4_tiled<2, 1>(p, st);
-  if (rc != ARCQ_OK) return rc;
-  const size_t total4 = ((size_t)p.M * p.N) >> 2;
-  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<size_t>((total4 + 255) / 256, 1024)), dim3(256), 0, st, p);
-  ARCQ_HIP_TRY(hipGetLastError());
-  return ARCQ_OK;
-}
-
-}  // namespace
-}  // namespace arcq
-
-static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
-                       int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b,
-                       const void *residual, void *c, void *stream);
-
-extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
-                           int M, int N, int Kp, int fmt, float alpha, const float *d_alpha_a,
-                           const float *d_alpha_b, void *c, void *stream) {
-  return matmul_impl(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b, nullptr, c, stream);
-}
-
-extern "C" int arcq_matmul_add(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
-                               int M, int N, int Kp, int fmt, float alpha, const float *d_alpha_a,
-                               const float *d_alpha_b, const void *residual, void *c, void *stream) {
-  if (!residual) return ARCQ_ERR_NULL;
-  if (!arcq::aligned16(residual)) return ARCQ_ERR_ALIGN;
-  return matmul_impl(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b, residual, c, stream);
-}
-
-static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
-                       int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b,
-                       const void *residual, void *c, void *stream) {
-  using namespace arcq;
-  if (fmt != ARCQ_FMT_NVFP4 && fmt != ARCQ_FMT_MXFP4) return ARCQ_ERR_FORMAT;
-  if (M < 0 || N < 0 || Kp < 64 || Kp % 64 != 0) return ARCQ_ERR_SHAPE;
-  if (M == 0 || N == 0) return ARCQ_OK;
-  if (!a_codes || !a_scales || !b_codes || !b_scales || !c) return ARCQ_ERR_NULL;
-  if (!aligned16(a_codes) || !aligned16(b_codes) || !aligned16(c)) return ARCQ_ERR_ALIGN;
-  GemmParams p;
-  p.a_codes = static_cast<const uint8_t *>(a_codes);
-  p.a_scales = static_cast<const uint8_t *>(a_scales);
-  p.b_codes = static_cast<const uint8_t *>(b_codes);
-  p.b_scales = static_cast<const uint8_t *>(b_scales);
-  p.c = static_cast<uint16_t *>(c);
-  p.d_alpha_a = d_alpha_a;
-  p.d_alpha_b = d_alpha_b;
-  p.alpha = alpha;
-  p.M = M;
-  p.N = N;
-  p.Kp = Kp;
-  p.residual = static_cast<const uint16_t *>(residual);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  dim3 grid((N + kWgN - 1) / kWgN, (M + kWgM - 1) / kWgM);
-  // Tile choice (ARCQ_GEMM_KERNEL=<WN><WM> forces one, 0 forces the direct kernels; for tuning):
-  // few rows of activations -> small tiles so that enough workgroups exist; many -> large tiles
-  // for operand reuse.  K' % 128 != 0 goes to the direct kernels.
-  static const int force = getenv("ARCQ_GEMM_KERNEL") ? atoi(getenv("ARCQ_GEMM_KERNEL")) : -1;
-  static const int skinny_max = getenv("ARCQ_GEMM_SKINNY_MAX") ? atoi(getenv("ARCQ_GEMM_SKINNY_MAX")) : 64;
-  const bool fast_ok = Kp % 128 == 0 && aligned16(a_scales) && aligned16(b_scales);
+GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
+  GemmPlan plan;
+  const Tuning &tune = tuning();
+  const int force = tune.gemm_kernel, split_env = tune.gemm_splitk;
+  const bool fast_ok = Kp % 128 == 0 && scales_aligned;
   // Measured crossover against the tiled kernels (weights streaming from HBM): the skinny kernels
   // re-read the activations from L2 once per 16 weight rows, which costs more the larger M and N are.
   const bool skinny_wins = fmt == ARCQ_FMT_MXFP4
@@ -1093,8 +1026,6 @@ static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_
   // Narrow layers with a decode batch of tens of rows: 128x64 tiles with K cut into slices (measured
   // against the skinny and the plain tiled kernels with the weights streaming from HBM; two launches,
   // so it pays only where the single launch is far from the weight stream's time).
-  // ARCQ_GEMM_SPLITK=<slices> forces it for M <= 64, =1 switches it off.
-  static const int split_env = getenv("ARCQ_GEMM_SPLITK") ? atoi(getenv("ARCQ_GEMM_SPLITK")) : 0;
   int split = 0;
   bool one_round_21 = false;  // 128x64 tiles, no more of them than CUs, K not cut
   if (split_env > 1) split = M <= 512 ? split_env : 0;
@@ -1115,12 +1046,17 @@ static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_
   }
   if (split > 1 && fast_ok && Kp >= 512 && (N & 3) == 0) {
     const int slices = std::min(split, (Kp + 255) / 256 / 2);
-    const int rc = fmt == ARCQ_FMT_MXFP4 ? launch_tiled_splitk<ARCQ_FMT_MXFP4>(p, slices, st)
-                                         : launch_tiled_splitk<ARCQ_FMT_NVFP4>(p, slices, st);
-    if (rc >= 0) return rc;
+    const size_t bytes = (size_t)slices * M * N * sizeof(float);
+    if (slices > 1 && bytes <= kSplitMaxBytes) {
+      plan.kernel = fmt == ARCQ_FMT_MXFP4 ? 214 : 21;
+      plan.slices = slices;
+      plan.scratch = bytes;
+      return plan;
+    }
   }
-  if (fast_ok && (force == 1 || (force < 0 && M <= skinny_max && skinny_wins)) && M <= 64) {
-    return fmt == ARCQ_FMT_MXFP4 ? launch_skinny_for<ARCQ_FMT_MXFP4>(p, st) : launch_skinny_for<ARCQ_FMT_NVFP4>(p, st);
+  if (fast_ok && (force == 1 || (force < 0 && skinny_wins)) && M <= 64) {
+    plan.kernel = 1;
+    return plan;
   }
   // the tiled kernels fetch scale bytes in 16-byte windows that are shifted back at the end of a row:
   // the row must be at least one window long (K' >= 512 for MXFP4, 256 for NVFP4)
@@ -1143,25 +1079,116 @@ static int matmul_impl(const void *a_codes, const void *a_scales, const void *b_
                                               : (M <= 128 ? 21
                                                           : (M < 512 ? 22
                                                                      : (c44 < c42 && c44 < c22 ? 44 : (c42 <= c22 ? 42 : 22)))));
-    if (force == 44 || (force < 0 && pick == 44)) return launch_mxfp4_tiled<4, 4>(p, st);
-    if (force == 42 || (force < 0 && pick == 42)) return launch_mxfp4_tiled<4, 2>(p, st);
-    if (force == 24) return launch_mxfp4_tiled<2, 4>(p, st);
-    if (force == 224 || (force < 0 && pick == 224)) return launch_mxfp4_tiled<2, 2, 4>(p, st);
-    if (force == 22 || (force < 0 && pick == 22)) return launch_mxfp4_tiled<2, 2>(p, st);
-    if (force == 214 || (force < 0 && pick == 214)) return launch_mxfp4_tiled<2, 1, 4>(p, st);
-    if (force == 21 || force < 0) return launch_mxfp4_tiled<2, 1>(p, st);
+    plan.kernel = force > 1 ? force : pick;
+    return plan;
   }
   if (fmt == ARCQ_FMT_NVFP4 && force != 0 && tiled_ok) {
-    if (force == 44 || (force < 0 && M > 1024)) return launch_nvfp4_tiled<4, 4>(p, st);
-    if (force == 42) return launch_nvfp4_tiled<4, 2>(p, st);
-    if (force == 34) return launch_nvfp4_tiled<3, 4>(p, st);
-    if (force == 22 || (force < 0 && M > 128 && !one_round_21)) return launch_nvfp4_tiled<2, 2>(p, st);
-    if (force == 21 || force < 0) return launch_nvfp4_tiled<2, 1>(p, st);
+    plan.kernel = force > 1 ? force : (M > 1024 ? 44 : (M > 128 && !one_round_21 ? 22 : 21));
+    return plan;
   }
+  plan.kernel = 0;
+  return plan;
+}
+
+int run_gemm(GemmParams p, const GemmPlan &plan, int fmt, float *scratch, hipStream_t st) {
+  if (plan.slices > 1) {
+    p.k_slices = plan.slices;
+    p.partial = scratch;
+    const int rc = fmt == ARCQ_FMT_MXFP4 ? launch_mxfp4_tiled<2, 1, 4>(p, st) : launch_nvfp4_tiled<2, 1>(p, st);
+    if (rc != ARCQ_OK) return rc;
+    const size_t total4 = ((size_t)p.M * p.N) >> 2;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<size_t>((total4 + 255) / 256, 1024)), dim3(256), 0,
+                       st, p);
+    ARCQ_HIP_TRY(hipGetLastError());
+    return ARCQ_OK;
+  }
+  if (plan.kernel == 1)
+    return fmt == ARCQ_FMT_MXFP4 ? launch_skinny_for<ARCQ_FMT_MXFP4>(p, st) : launch_skinny_for<ARCQ_FMT_NVFP4>(p, st);
+  if (fmt == ARCQ_FMT_MXFP4) {
+    switch (plan.kernel) {
+      case 44: return launch_mxfp4_tiled<4, 4>(p, st);
+      case 42: return launch_mxfp4_tiled<4, 2>(p, st);
+      case 224: return launch_mxfp4_tiled<2, 2, 4>(p, st);
+      case 22: return launch_mxfp4_tiled<2, 2>(p, st);
+      case 214: return launch_mxfp4_tiled<2, 1, 4>(p, st);
+      case 21: return launch_mxfp4_tiled<2, 1>(p, st);
+      default: break;
+    }
+  } else {
+    switch (plan.kernel) {
+      case 44: return launch_nvfp4_tiled<4, 4>(p, st);
+      case 42: return launch_nvfp4_tiled<4, 2>(p, st);
+      case 22: return launch_nvfp4_tiled<2, 2>(p, st);
+      case 21: return launch_nvfp4_tiled<2, 1>(p, st);
+      default: break;
+    }
+  }
+  const dim3 grid((p.N + kWgN - 1) / kWgN, (p.M + kWgM - 1) / kWgM);
   if (fmt == ARCQ_FMT_MXFP4)
     hipLaunchKernelGGL(gemm_mxfp4_direct, grid, dim3(256), 0, st, p);
   else
     hipLaunchKernelGGL(gemm_nvfp4_direct, grid, dim3(256), 0, st, p);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
+}
+
+// argument checks shared by the entry points; fills p
+int check_gemm_args(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
+                    int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b, const void *residual,
+                    void *c, GemmParams *p) {
+  if (fmt != ARCQ_FMT_NVFP4 && fmt != ARCQ_FMT_MXFP4) return ARCQ_ERR_FORMAT;
+  if (M < 0 || N < 0 || Kp < 64 || Kp % 64 != 0) return ARCQ_ERR_SHAPE;
+  if (M == 0 || N == 0) return ARCQ_OK;
+  if (!a_codes || !a_scales || !b_codes || !b_scales || !c) return ARCQ_ERR_NULL;
+  if (!aligned16(a_codes) || !aligned16(b_codes) || !aligned16(c)) return ARCQ_ERR_ALIGN;
+  p->a_codes = static_cast<const uint8_t *>(a_codes);
+  p->a_scales = static_cast<const uint8_t *>(a_scales);
+  p->b_codes = static_cast<const uint8_t *>(b_codes);
+  p->b_scales = static_cast<const uint8_t *>(b_scales);
+  p->c = static_cast<uint16_t *>(c);
+  p->d_alpha_a = d_alpha_a;
+  p->d_alpha_b = d_alpha_b;
+  p->alpha = alpha;
+  p->M = M;
+  p->N = N;
+  p->Kp = Kp;
+  p->residual = static_cast<const uint16_t *>(residual);
+  return ARCQ_OK;
+}
+
+int matmul_impl(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
+                int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b, const void *residual,
+                void *c, void *stream) {
+  GemmParams p;
+  const int rc = check_gemm_args(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b,
+                                 residual, c, &p);
+  if (rc != ARCQ_OK || M == 0 || N == 0) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const GemmPlan plan = plan_gemm(M, N, Kp, fmt, aligned16(a_scales) && aligned16(b_scales));
+  float *scratch = nullptr;
+  if (plan.slices > 1) {
+    int status = ARCQ_OK;
+    scratch = static_cast<float *>(stream_workspace(kWsSplitK, st, &status));
+    if (!scratch) return status;
+  }
+  return run_gemm(p, plan, fmt, scratch, st);
+}
+
+}  // namespace
+}  // namespace arcq
+
+extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                           int M, int N, int Kp, int fmt, float alpha, const float *d_alpha_a,
+                           const float *d_alpha_b, void *c, void *stream) {
+  return arcq::matmul_impl(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b, nullptr, c,
+                           stream);
+}
+
+extern "C" int arcq_matmul_add(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                               int M, int N, int Kp, int fmt, float alpha, const float *d_alpha_a,
+                               const float *d_alpha_b, const void *residual, void *c, void *stream) {
+  if (!residual) return ARCQ_ERR_NULL;
+  if (!arcq::aligned16(residual)) return ARCQ_ERR_ALIGN;
+  return arcq::matmul_impl(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b, residual, c,
+                           stream);
 }

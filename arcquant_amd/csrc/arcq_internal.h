@@ -20,5 +20,36 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
     if (_e != hipSuccess) return ::arcq::note_hip_error(_e); \
   } while (0)
 
+// Scratch memory of the kernels that need some beyond their inputs and outputs.  One buffer per
+// (device, stream, kind), allocated on the first call that needs it (or by arcq_prepare_stream) and
+// kept until the process ends, so that a captured graph may hold its address.  Work on one stream is
+// serialised, so two calls never share a buffer unless they share a stream.
+enum WorkspaceKind {
+  kWsTensorScale = 0,  // running maximum + arrival counter of arcq_tensor_scale (zeroed once)
+  kWsSplitK = 1,       // fp32 partial tiles of the split-K GEMM
+  kWsDecode = 2,       // partial softmax sums of the split decode attention
+  kWsKinds = 3
+};
+constexpr size_t kWorkspaceBytes[kWsKinds] = {256, 32u << 20, 8u << 20};
+
+// The buffer of `kind` for (current device, stream).  Returns nullptr and sets *status when there is
+// none and none can be made: ARCQ_ERR_WORKSPACE while `stream` is capturing (an allocation there
+// would break the capture), ARCQ_ERR_LAUNCH when the allocation fails.
+void *stream_workspace(int kind, hipStream_t stream, int *status);
+
+// Overrides for tuning runs, read from the environment once, when the library is first used:
+//   ARCQ_GEMM_KERNEL=<WN><WM>   force a GEMM tile (44, 42, 22, 21; 214 / 224 = four-stage ring; 1 = skinny, 0 = direct)
+//   ARCQ_GEMM_SPLITK=<slices>   force split-K for M <= 512 (1 = never split)
+//   ARCQ_QUANT_GRID=<n>         workgroups of the row quantizers
+//   ARCQ_KV_DECODE_SPLITS=<n>   ranges per sequence of the decode attention
+// Unset (the normal case) every field keeps the value below and the dispatch is the measured one.
+struct Tuning {
+  int gemm_kernel = -1;
+  int gemm_splitk = 0;
+  int quant_grid = 0;
+  int kv_decode_splits = 0;
+};
+const Tuning &tuning();
+
 }  // namespace arcq
 #endif  // ARCQ_INTERNAL_H_

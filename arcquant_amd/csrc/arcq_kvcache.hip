@@ -19,7 +19,6 @@
 #include <stdlib.h>
 
 #include <algorithm>
-#include <mutex>
 #include <type_traits>
 
 #include "../../include/arcq.h"
@@ -240,6 +239,7 @@ __global__ __launch_bounds__(256) void kv_append_i4_kernel(const uint16_t *k, co
   for (int r = blockIdx.y * 16 + (threadIdx.x >> 4); r < rows; r += gridDim.y * 16) {
     const int i = r / c.heads, head = r - i * c.heads;
     const int pos = len - n_new + i;
+    if (np <= 0 || pos < 0 || pos >= np * c.page_size) continue;  // a table without room for this token: no store
     const int page = c.indices[p0 + pos / c.page_size], slot = pos % c.page_size;
     const size_t src = ((size_t)(tok0 + i) * c.heads + head) * kHeadDim;
     quantize_row_store<BF16>(k + src, c, kv_row(c, page, 0, head, slot), lane16);
@@ -261,6 +261,7 @@ __global__ __launch_bounds__(256) void kv_store_i4_kernel(const uint32_t *kq, co
   for (int r = blockIdx.y * 16 + (threadIdx.x >> 4); r < rows; r += gridDim.y * 16) {
     const int i = r / c.heads, head = r - i * c.heads;
     const int pos = len - n_new + i;
+    if (np <= 0 || pos < 0 || pos >= np * c.page_size) continue;  // a table without room for this token: no store
     const int page = c.indices[p0 + pos / c.page_size], slot = pos % c.page_size;
     const size_t src = (size_t)(tok0 + i) * c.heads + head;
     const size_t krow = kv_row(c, page, 0, head, slot), vrow = kv_row(c, page, 1, head, slot);
@@ -454,6 +455,8 @@ constexpr int kDecodeWaves = 8;
 // flight, each wave into its own slots: codes of K (1 KB), codes of V (1 KB), the 32 parameter words.
 constexpr int kDecodeStages = 4;
 constexpr int kDecodeSlotBytes = 1024 + 1024 + 128;
+// These write M0, which the compiler reserves and does not accept on a clobber list: the decode kernel
+// holds nothing for which the compiler sets or reads M0 itself, and each helper sets it before its load.
 __device__ __forceinline__ void kv_lds_dma16(const void *g, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_wave_base), "v"(g) : "memory");
 }
@@ -711,25 +714,6 @@ __global__ __launch_bounds__(128) void kv_decode_merge_kernel(uint16_t *o, const
   o[(size_t)blockIdx.x * kHeadDim + threadIdx.x] = (uint16_t)to_bits<BF16>(out);
 }
 
-// partials of the split decode: one buffer per device, allocated on first use and kept
-constexpr size_t kDecodeWorkspaceBytes = 8u << 20;
-inline float *decode_workspace() {
-  static std::mutex mu;
-  static float *ws[16];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
-  std::lock_guard<std::mutex> lock(mu);
-  if (!ws[dev]) {
-    float *w = nullptr;
-    if (hipMalloc(&w, kDecodeWorkspaceBytes) != hipSuccess) {
-      (void)hipGetLastError();
-      return nullptr;
-    }
-    ws[dev] = w;
-  }
-  return ws[dev];
-}
-
 int check_layout(const void *kv_data, const void *kv_param, const int32_t *kv_indptr, const int32_t *kv_indices,
                  const int32_t *last_page_offset, int n_layers, int layer_idx, int heads, int page_size, int head_dim,
                  int dtype) {
@@ -882,25 +866,28 @@ int arcq_kv_decode_i4(void *o, const void *q, int dtype, int batch, int num_qo_h
              num_kv_heads,
              page_size};
   const float sl2 = sm_scale * 1.4426950408889634f;
-  static const bool force_valu = getenv("ARCQ_KV_DECODE_VALU") != nullptr;
-  static const int split_env = getenv("ARCQ_KV_DECODE_SPLITS") ? atoi(getenv("ARCQ_KV_DECODE_SPLITS")) : 0;
-  const bool mfma = page_size % 16 == 0 && !force_valu;
+  const bool mfma = page_size % 16 == 0;
   // few (sequence, KV head) pairs: cut the sequences so that about two workgroups per CU exist (the
-  // lengths live on the device, so the cut is by count only; a range without tokens costs nothing)
+  // lengths live on the device, so the cut is by count only; a range without tokens costs nothing).
+  // The ranges' partial sums go through the stream's scratch buffer.
+  hipStream_t st = static_cast<hipStream_t>(stream);
   int splits = 1;
   float *partial = nullptr;
   if (mfma) {
     const long pairs = (long)batch * num_kv_heads;
+    const int split_env = tuning().kv_decode_splits;
     splits = split_env > 0 ? split_env : (pairs >= 256 ? 1 : (int)((512 + pairs - 1) / pairs));
     if (splits > 16) splits = 16;
+    if (splits > 1 &&
+        (size_t)batch * num_qo_heads * splits * kPartialStride * sizeof(float) > kWorkspaceBytes[kWsDecode])
+      splits = 1;
     if (splits > 1) {
-      partial = decode_workspace();
-      if (!partial || (size_t)batch * num_qo_heads * splits * kPartialStride * sizeof(float) > kDecodeWorkspaceBytes)
-        splits = 1;
+      int status = ARCQ_OK;
+      partial = static_cast<float *>(stream_workspace(kWsDecode, st, &status));
+      if (!partial) return status;
     }
   }
   dim3 grid(batch, num_kv_heads, splits);
-  hipStream_t st = static_cast<hipStream_t>(stream);
   uint16_t *op = static_cast<uint16_t *>(o);
   const uint16_t *qp = static_cast<const uint16_t *>(q);
 #define ARCQ_LAUNCH_DECODE(BF, GG)                                                                                \

@@ -7,10 +7,6 @@
 // reordered channels ("unit"): a whole NVFP4 block, or half an MXFP4 block whose other half
 // sits in the neighbouring lane (one cross-lane max).
 #include <hip/hip_runtime.h>
-#include <stdlib.h>
-
-#include <mutex>
-
 #include "arcq_internal.h"
 #include "arcq_math.h"
 
@@ -718,29 +714,6 @@ __global__ __launch_bounds__(256) void tensor_scale_kernel(const uint16_t *x, co
   atomicExch(ws + 1, 0u);
 }
 
-// the two workspace words, one pair per device, allocated (and zeroed) on first use and kept
-inline uint32_t *tensor_scale_workspace() {
-  static std::mutex mu;
-  static uint32_t *ws[16];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
-  std::lock_guard<std::mutex> lock(mu);
-  if (!ws[dev]) {
-    uint32_t *w = nullptr;
-    if (hipMalloc(&w, 2 * sizeof(uint32_t)) != hipSuccess) {
-      (void)hipGetLastError();
-      return nullptr;
-    }
-    if (hipMemset(w, 0, 2 * sizeof(uint32_t)) != hipSuccess) {
-      (void)hipGetLastError();
-      (void)hipFree(w);
-      return nullptr;
-    }
-    ws[dev] = w;
-  }
-  return ws[dev];
-}
-
 template <int FMT, int MODE, bool SCALED>
 int launch_quantize_unit(const QuantParams &p, hipStream_t stream) {
   const int threads = (((p.K >> 4) + 63) / 64) * 64;
@@ -749,7 +722,7 @@ int launch_quantize_unit(const QuantParams &p, hipStream_t stream) {
   // the kernel's register count lets 4 waves per SIMD (16 per CU) be resident: launch exactly the
   // resident workgroups so that each amortises its set-up over as many rows as possible
   int grid = 256 * (16 / waves_per_wg > 0 ? 16 / waves_per_wg : 1);
-  if (const char *e = getenv("ARCQ_QUANT_GRID")) grid = atoi(e);
+  if (tuning().quant_grid > 0) grid = tuning().quant_grid;
   if (grid > p.rows) grid = p.rows;
   hipLaunchKernelGGL((quantize_rows_unit_kernel<FMT, MODE, SCALED>), dim3(grid), dim3(threads), lds, stream, p);
   ARCQ_HIP_TRY(hipGetLastError());
@@ -858,7 +831,7 @@ int quantize_entry(int mode, const void *x, const void *gamma, float eps, int ro
     return launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_NORM, false>(p, st);
   }
   // any other tensor scale, on the host or on the device: same kernel with the two-sided encode
-  if (mode != MODE_NORM && K <= 16384 && !getenv("ARCQ_QUANT_GENERIC")) {
+  if (mode != MODE_NORM && K <= 16384) {
     if (fmt == ARCQ_FMT_NVFP4) {
       if (mode == MODE_X) return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_X, true>(p, st);
       return launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_W, true>(p, st);
@@ -989,12 +962,13 @@ int arcq_tensor_scale(const void *x, const void *up, int ld, int M, int K, float
   if (M < 0 || K < 8 || K % 8 != 0 || ld < K || ld % 8 != 0 || !(divisor > 0.0f)) return ARCQ_ERR_SHAPE;
   if (!x || !d_scale) return ARCQ_ERR_NULL;
   if (!arcq::aligned16(x) || (up && !arcq::aligned16(up))) return ARCQ_ERR_ALIGN;
-  uint32_t *ws = arcq::tensor_scale_workspace();
-  if (!ws) return ARCQ_ERR_LAUNCH;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int status = ARCQ_OK;
+  uint32_t *ws = static_cast<uint32_t *>(arcq::stream_workspace(arcq::kWsTensorScale, st, &status));
+  if (!ws) return status;
   const size_t chunks = (size_t)M * (K >> 3);
   int grid = (int)((chunks + 1023) / 1024 < 1024 ? (chunks + 1023) / 1024 : 1024);  // four chunks per thread
   if (grid < 1) grid = 1;  // M == 0: one block writes the scale of an empty tensor, 1
-  hipStream_t st = static_cast<hipStream_t>(stream);
   if (up)
     hipLaunchKernelGGL(arcq::tensor_scale_kernel<true>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(x),
                        static_cast<const uint16_t *>(up), (size_t)ld, M, K, divisor, ws, d_scale);

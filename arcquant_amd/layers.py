@@ -275,8 +275,19 @@ class LlamaAttention(nn.Module):
             kc[:, :, past_len:past_len + q_len] = k
             vc[:, :, past_len:past_len + q_len] = v
             k, v = kc[:, :, :past_len + q_len], vc[:, :, :past_len + q_len]
-        out = F.scaled_dot_product_attention(q, k, v, is_causal=(q_len > 1 and past_len == 0),
-                                             enable_gqa=(nkv != nh))
+        if q_len == 1:
+            mask, causal = None, False
+        elif isinstance(past_len, int) and past_len == 0:
+            mask, causal = None, True
+        elif isinstance(past_len, int):
+            # a chunk of new tokens behind past_len cached ones: new token i sees the cache and the new
+            # tokens up to itself (the lower-right aligned mask of model/qLlamaLayer.py's attention_mask)
+            total = past_len + q_len
+            mask = torch.ones(q_len, total, dtype=torch.bool, device=q.device).tril(diagonal=past_len)
+            causal = False
+        else:
+            raise RuntimeError("a device-side past_len (graph replay) is for decode steps: one new token per sequence")
+        out = F.scaled_dot_product_attention(q, k, v, attn_mask=mask, is_causal=causal, enable_gqa=(nkv != nh))
         out = out.transpose(1, 2).reshape(bsz, q_len, nh * d)
         return self.o_proj(quantize_tokens(out, self.o_reorder_index, self.o_proj.select_num, self.quant_type), residual)
 
@@ -404,25 +415,34 @@ class GraphedDecodeStep:
     """One decoder layer's decode step (one new token per sequence, INT4 paged KV cache) captured
     once as a HIP graph and replayed: the step is a chain of ~20 short launches whose issue cost on
     the host exceeds their run time.  Host-side cache bookkeeping happens in cache.begin_step() before
-    each replay; the token positions for the rotary embedding are read from cache.positions on the
-    device.  No memset nodes are recorded (buffers are cleared by fill kernels)."""
+    the replay; the token positions for the rotary embedding are read from cache.positions on the
+    device.  No memset nodes are recorded (buffers are cleared by fill kernels).
 
-    def __init__(self, layer: LlamaDecoderLayer, cache, batch, hidden, layer_idx=0, warmup=3):
+    The cache is shared by all layers of a model and must advance once per token, not once per layer:
+    only the step with ``advance=True`` (the default for layer_idx 0) calls cache.begin_step(); the steps
+    of the other layers run behind it on the advanced cache.  A caller that advances the cache itself
+    passes advance=False everywhere."""
+
+    def __init__(self, layer: LlamaDecoderLayer, cache, batch, hidden, layer_idx=0, warmup=3, advance=None):
         self.layer, self.cache, self.layer_idx = layer, cache, layer_idx
+        self.advance = (layer_idx == 0) if advance is None else bool(advance)
         cache.external_step = True
         self.x = torch.zeros(batch, 1, hidden, dtype=torch.bfloat16, device=cache.device)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         saved = list(cache.lengths)
+        # warm-up and capture run on a cache advanced by one token (the slot a real step writes), whichever
+        # layer this is; the cache is put back afterwards, and the slot is rewritten by the first real step
         with torch.cuda.stream(side):            # warm-up on a side stream, as graph capture requires
-            for _ in range(warmup):
+            agemm.prepare_stream(cache.device)   # the library's scratch buffers belong to a stream: the capture
+            for _ in range(warmup):              # below runs on this same stream and finds them allocated
                 cache.begin_step()
                 self._run()
                 self._rewind(saved)
         torch.cuda.current_stream().wait_stream(side)
         cache.begin_step()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        with torch.cuda.graph(self.graph, stream=side):
             self.y = self._run()
         self._rewind(saved)
 
@@ -435,7 +455,8 @@ class GraphedDecodeStep:
 
     @torch.no_grad()
     def __call__(self, hidden_states):
-        self.cache.begin_step()
+        if self.advance:
+            self.cache.begin_step()
         if hidden_states.data_ptr() != self.x.data_ptr():    # a caller may write into self.x directly
             self.x.copy_(hidden_states)
         self.graph.replay()

@@ -39,7 +39,9 @@ typedef enum {
   ARCQ_ERR_FORMAT = 3,   /* fmt is neither ARCQ_FMT_NVFP4 nor ARCQ_FMT_MXFP4 */
   ARCQ_ERR_ALIGN = 4,    /* a pointer is not 16-byte aligned */
   ARCQ_ERR_LAUNCH = 5,   /* the HIP runtime refused the launch (see arcq_last_hip_error) */
-  ARCQ_ERR_INDEX = 6     /* reorder_index is not a permutation of 0..K-1 (arcq_check_index) */
+  ARCQ_ERR_INDEX = 6,    /* reorder_index is not a permutation of 0..K-1 (arcq_check_index) */
+  ARCQ_ERR_WORKSPACE = 7 /* scratch memory unavailable: the stream is being captured and has none yet
+                            (arcq_prepare_stream), or the problem exceeds a fixed scratch buffer */
 } arcq_status;
 
 enum { ARCQ_FMT_NVFP4 = 0, ARCQ_FMT_MXFP4 = 1 };
@@ -49,6 +51,21 @@ int arcq_version(void);
 const char *arcq_status_string(int status);
 /* hipError_t of the last failed launch on this thread, as an int (0 = none). */
 int arcq_last_hip_error(void);
+
+/*
+ * Scratch memory.  Three kernels need device memory beyond their inputs and outputs: the split-K GEMM
+ * (fp32 partial tiles, arcq_matmul on narrow layers with few rows), the split decode attention
+ * (partial softmax sums, arcq_kv_decode_i4 with few sequences) and arcq_tensor_scale (two words).
+ * The library keeps one buffer of each kind per (device, stream), allocated on the first call that
+ * needs it and never freed; calls on one stream are serialised, so they never share a buffer with a
+ * call on another stream.  An allocation cannot happen while the stream is being captured into a
+ * graph: such a call returns ARCQ_ERR_WORKSPACE unless the stream has its buffers already.
+ * arcq_prepare_stream allocates all three for (current device, stream) -- call it once before
+ * capturing on that stream.  A graph replayed on another stream still uses the buffers of the stream
+ * it was captured on.  (The reference keeps no state between calls: its CUTLASS GEMM has no split-K
+ * and it computes tensor scales with torch, kernels/src/nvfp4.cu:35-132, model/qLlamaLayer.py:73-77.)
+ */
+int arcq_prepare_stream(void *stream);
 
 /* Block size G of a format (16 / 32), or 0 for an unknown format. */
 int arcq_group_size(int fmt);
@@ -127,8 +144,7 @@ int arcq_swiglu_absmax(const void *gate, const void *up, int ld, int M, int K, f
  *   up       NULL, or the second operand of a fused SwiGLU: the scale is then that of
  *            act_fn(x) * up (x = gate), as arcq_swiglu_quantize_x forms it
  *   d_scale  fp32 scalar on the device, read by the quantizer (d_global_scale) and the GEMM (d_alpha_a)
- * Blocks combine their maxima through two words of a per-device workspace that the library allocates
- * on first use and keeps; calls that overlap in time on one device would share it.
+ * Blocks combine their maxima through two words of the stream's scratch memory (arcq_prepare_stream).
  */
 int arcq_tensor_scale(const void *x, const void *up, int ld, int M, int K, float divisor, float *d_scale, void *stream);
 

@@ -43,6 +43,16 @@ def build(force: bool = False) -> str:
     return _LIB_PATH
 
 
+def build_hostmath(force: bool = False) -> str:
+    """Compile host_math.cpp: the kernels' scalar arithmetic (arcquant_amd/csrc/arcq_math.h) built for the host
+    with the exhaustive checks of its shortcuts.  Test scaffolding, like the rest of this package."""
+    path = os.path.join(_HERE, "libarcq_hostmath.so")
+    deps = [os.path.join(_HERE, "host_math.cpp"), os.path.join(_HERE, "..", "arcquant_amd", "csrc", "arcq_math.h")]
+    if force or not os.path.exists(path) or any(os.path.getmtime(path) < os.path.getmtime(d) for d in deps):
+        subprocess.check_call(["make", "-s", "-C", _HERE, "-B", "libarcq_hostmath.so"])
+    return path
+
+
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:

@@ -286,3 +286,69 @@ def test_rope_rows_match_torch(kvc, dtype):
     k = wide[:, nh * 128:(nh + nkv) * 128].view(-1, nkv, 128)
     assert torch.equal(q_rot.cpu(), q * cos + rot(q) * sin)
     assert torch.equal(k_rot.cpu(), k * cos + rot(k) * sin)
+
+
+@pytest.mark.parametrize("name,dtype", [("f16", torch.float16), ("bf16", torch.bfloat16)])
+def test_quantize_append_matches_reference_vectors(kvc, ref, name, dtype):
+    """the fused quantize + append on the inputs of the reference-written vectors
+    (tests/golden/refkv_golden.npz, from model/kv_cache.py:21-37): codes, scales and zeros as the
+    reference's own function returned them"""
+    import os
+    import numpy as np
+    gold = dict(np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "refkv_golden.npz"),
+                        allow_pickle=False))
+    x = torch.from_numpy(gold[f"{name}_x_bits"]).view(dtype)           # [12 tokens, 8 heads, 128]
+    tokens, heads, _ = x.shape
+    page_size = 4
+    indptr, indices, last, maxc = make_table([tokens], page_size, 1)
+    pages = torch.zeros(maxc, 1, 2, heads, page_size, 64, dtype=torch.uint8, device="cuda")
+    params = torch.zeros(maxc, 1, 2, heads, page_size, 2, dtype=dtype, device="cuda")
+    seq = torch.tensor([0, tokens], dtype=torch.int32).cuda()
+    print(f"kv append, reference vectors, {name}", flush=True)
+    kvc.quantize_append(pages, params, indptr.cuda(), indices.cuda(), last.cuda(), x.cuda(), x.flip(0).contiguous().cuda(), 0,
+                        seqlen_indptr=seq)
+    (kc, kp), (vc, vp) = ref.gather_sequence(pages.cpu(), params.cpu(), indptr, indices, last, 0, 0)
+    want_q = ref.unpack(torch.from_numpy(gold[f"{name}_q"]))
+    want_s = torch.from_numpy(gold[f"{name}_scale_bits"]).view(dtype).double()[..., 0]
+    want_z = torch.from_numpy(gold[f"{name}_zero_bits"]).view(dtype).double()[..., 0]
+    assert torch.equal(kc, want_q) and torch.equal(vc, want_q.flip(0))
+    assert torch.equal(kp[..., 0], want_s) and torch.equal(kp[..., 1], want_z)
+    assert torch.equal(vp[..., 0], want_s.flip(0)) and torch.equal(vp[..., 1], want_z.flip(0))
+
+
+def test_inconsistent_page_table_stores_nothing(kvc):
+    """a sequence whose table has no page (or no room for its new tokens) must not be written anywhere:
+    the kernels skip such rows instead of indexing the page list out of range"""
+    heads, page_size = 2, 16
+    pages = torch.zeros(4, 1, 2, heads, page_size, 64, dtype=torch.uint8, device="cuda")
+    params = torch.zeros(4, 1, 2, heads, page_size, 2, dtype=torch.float16, device="cuda")
+    k = torch.randn(2, heads, 128).half().cuda()
+    # sequence 0 has no pages at all; sequence 1 owns page 2 and holds one token after the append
+    indptr = torch.tensor([0, 0, 1], dtype=torch.int32).cuda()
+    indices = torch.tensor([2], dtype=torch.int32).cuda()
+    last = torch.tensor([0, 1], dtype=torch.int32).cuda()
+    kvc.quantize_append(pages, params, indptr, indices, last, k, k, 0)
+    torch.cuda.synchronize()
+    assert int(pages[[0, 1, 3]].sum()) == 0 and float(params[[0, 1, 3]].abs().sum()) == 0
+    assert int(pages[2, 0, :, :, 0].sum()) > 0 and int(pages[2, 0, :, :, 1:].sum()) == 0
+    # the pre-quantized store takes the same table; three new tokens for a sequence that holds one: skipped rows
+    q = torch.full((4, heads, 64), 0x77, dtype=torch.uint8, device="cuda")
+    par = torch.ones(4, heads, 2, dtype=torch.float16, device="cuda")
+    pages.zero_()
+    seq = torch.tensor([0, 1, 4], dtype=torch.int32).cuda()
+    kvc.init_kv_i4(pages, params, indptr, indices, last, q, q, par, par, seq, 0)
+    torch.cuda.synchronize()
+    assert int(pages[[0, 1, 3]].sum()) == 0
+    assert int(pages[2, 0, :, :, 1:].sum()) == 0                       # only slot 0 (the token that fits) is written
+
+
+def test_agemm_module_exports_the_kv_operators():
+    """the reference reaches the KV operators through its extension module (kernels/src/bindings.cpp:576-578,
+    model/kv_cache.py:49-80): the drop-in module carries the same three names"""
+    from arcquant_amd import agemm, kv_cache
+    for name in ("init_kv_i4", "append_kv_i4", "batch_decode_i4"):
+        assert getattr(agemm, name) is getattr(kv_cache, name)
+    ns = {}
+    exec("from arcquant_amd.agemm import *", ns)
+    assert {"matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "init_kv_i4", "append_kv_i4",
+            "batch_decode_i4"} <= set(ns)

@@ -195,3 +195,54 @@ def test_graphed_decode_step_matches_eager(layers, fmt):
         assert graph_cache.lengths == eager_cache.lengths
         assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
     assert torch.equal(graph_cache.pages, eager_cache.pages) and torch.equal(graph_cache.scales, eager_cache.scales)
+
+
+def test_graphed_decode_steps_of_two_layers_share_one_cache(layers):
+    """Two decoder layers over one two-layer INT4 cache, one graphed step per layer: the cache advances
+    once per token (by the first layer's step), and every replay gives what the eager layers give."""
+    from arcquant_amd.kv_cache import MultiLayerPagedKVCache4Bit
+    fmt, hidden, inter, nh, nkv, S, batch, page = "MXFP4", 512, 1024, 4, 2, 64, 3, 16
+    model = [layers.LlamaDecoderLayer(hidden, inter, nh, nkv, select_num=S, select_num_down=S, quant_type=fmt, seed=20 + i)
+             for i in range(2)]
+    g = torch.Generator().manual_seed(21)
+    prompt = torch.randn(batch, 15, hidden, generator=g).to(torch.bfloat16).cuda()
+    caches = [MultiLayerPagedKVCache4Bit(batch, page, 64, "cuda", 2, nkv, 128, dtype=torch.bfloat16) for _ in range(2)]
+    for c in caches:
+        h = prompt
+        for i, layer in enumerate(model):
+            h = layer(h, c, 0, i)
+    eager_cache, graph_cache = caches
+    steps = [layers.GraphedDecodeStep(layer, graph_cache, batch, hidden, layer_idx=i) for i, layer in enumerate(model)]
+    assert graph_cache.lengths == [15] * batch
+    for t in range(4):                                              # lengths 15 -> 19: crosses a page boundary
+        x = torch.randn(batch, 1, hidden, generator=g).to(torch.bfloat16).cuda()
+        print(f"two-layer graphed decode, token {t}", flush=True)
+        pos = eager_cache.lengths[0]
+        want = x
+        for i, layer in enumerate(model):
+            want = layer(want, eager_cache, pos, i)
+        torch.cuda.synchronize()
+        got = x
+        for st in steps:
+            got = st(got)
+        got = got.clone()
+        torch.cuda.synchronize()
+        assert graph_cache.lengths == eager_cache.lengths == [16 + t] * batch
+        assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
+    assert torch.equal(graph_cache.pages, eager_cache.pages) and torch.equal(graph_cache.scales, eager_cache.scales)
+
+
+def test_chunked_prefill_is_causal(layers):
+    """q_len > 1 behind cached tokens over the bf16 (k, v) cache: the second chunk's outputs equal the
+    same rows of one full causal prefill (MXFP4: no tensor scale, so the two runs quantize alike)."""
+    hidden, inter, nh, nkv, S = 512, 1024, 4, 2, 64
+    layer = layers.LlamaDecoderLayer(hidden, inter, nh, nkv, select_num=S, select_num_down=S, quant_type="MXFP4", seed=31)
+    g = torch.Generator().manual_seed(32)
+    x = torch.randn(2, 24, hidden, generator=g).to(torch.bfloat16).cuda()
+    full = layer(x)
+    kv = (torch.zeros(2, nkv, 32, 128, dtype=torch.bfloat16, device="cuda"),
+          torch.zeros(2, nkv, 32, 128, dtype=torch.bfloat16, device="cuda"))
+    first = layer(x[:, :16].contiguous(), kv, 0)
+    second = layer(x[:, 16:].contiguous(), kv, 16)
+    assert rel_fro(first, full[:, :16]) < 2e-2
+    assert rel_fro(second, full[:, 16:]) < 2e-2

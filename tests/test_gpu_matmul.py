@@ -25,6 +25,13 @@ def rel_fro(got, want):
     return float((got - want).norm() / want.norm())
 
 
+def oracle_dq(oracle, codes, sf, fmt):
+    """fp32 values of codes + scale bytes from the CPU oracle's dequantizer, back on the GPU (the
+    library's own dequantizer stays out of the GEMM checks)"""
+    c = codes.cpu().numpy()
+    return torch.from_numpy(oracle.dequantize(c, sf.cpu().numpy().reshape(c.shape[0], -1), fmt)).cuda()
+
+
 def quantized_pair(agemm, M, N, K, S, fmt, seed):
     x = recipes.activations(M, K, seed=seed)
     w = recipes.weights(N, K, seed=seed + 1)
@@ -95,17 +102,17 @@ def test_identity_weights_recover_activations(agemm, oracle, fmt):
 @pytest.mark.parametrize("M,N,K,S", [(512, 4096, 4096, 256), (2048, 6144, 4096, 256), (256, 4096, 14336, 256),
                                      (512, 6144, 1024, 128), (448, 6200, 768, 256), (128, 28672, 1024, 256),
                                      (100, 4096, 4096, 256), (384, 4100, 8192, 128)])
-def test_matmul_llama_shapes_vs_torch_fp32(agemm, fmt, M, N, K, S):
+def test_matmul_llama_shapes_vs_torch_fp32(agemm, oracle, fmt, M, N, K, S):
     """Benchmark shapes, and shapes of one round of workgroups (at most 256 tiles of 128x64 or 128x128, also
     ragged and with K' % 256 == 128, and K cut into slices for a few hundred rows): compare with torch's
-    fp32 matmul of the dequantized operands on the GPU."""
+    fp32 matmul on the GPU of the operands as the CPU oracle dequantizes them."""
     (x, w, idx, gx, gw), (a, sfa, b, sfb) = quantized_pair(agemm, M, N, K, S, fmt, seed=3)
     print(f"matmul {fmt} M={M} N={N} K={K} S={S}", flush=True)
     y = agemm.matmul(a, b, sfa, sfb, gx * gw)
     prev = torch.backends.cuda.matmul.allow_tf32
     torch.backends.cuda.matmul.allow_tf32 = False
     try:
-        want = (agemm.dequantize(a, sfa, fmt=fmt) @ agemm.dequantize(b, sfb, fmt=fmt).T) * (gx * gw)
+        want = (oracle_dq(oracle, a, sfa, fmt) @ oracle_dq(oracle, b, sfb, fmt).T) * (gx * gw)
     finally:
         torch.backends.cuda.matmul.allow_tf32 = prev
     err = rel_fro(y.float(), want)
@@ -119,7 +126,7 @@ def test_matmul_llama_shapes_vs_torch_fp32(agemm, fmt, M, N, K, S):
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 32, 48, 64])
 @pytest.mark.parametrize("N,K,S", [(6144, 4096, 256), (202, 384, 0), (4100, 1024, 128), (4100, 8192, 128),
                                    (8324, 1024, 256), (8450, 768, 256)])
-def test_matmul_decode_batches(agemm, fmt, M, N, K, S):
+def test_matmul_decode_batches(agemm, oracle, fmt, M, N, K, S):
     """M <= 64 (decode batches) at a benchmark shape and at shapes whose N is not a multiple of the
     16-row strips or of the 4-wide stores: against torch's fp32 matmul of the dequantized operands,
     and, row by row, against the same call on a 128-row batch that contains these rows (another
@@ -137,7 +144,7 @@ def test_matmul_decode_batches(agemm, fmt, M, N, K, S):
     prev = torch.backends.cuda.matmul.allow_tf32
     torch.backends.cuda.matmul.allow_tf32 = False
     try:
-        want = (agemm.dequantize(a_m, sfa_m, fmt=fmt) @ agemm.dequantize(b, sfb, fmt=fmt).T) * (gx * gw)
+        want = (oracle_dq(oracle, a_m, sfa_m, fmt) @ oracle_dq(oracle, b, sfb, fmt).T) * (gx * gw)
     finally:
         torch.backends.cuda.matmul.allow_tf32 = prev
     assert rel_fro(y.float(), want) < TOL

@@ -7,12 +7,12 @@ import os
 import numpy as np
 import pytest
 
-from arcquant_amd import build as arcq_build
+import oracle as arcq_oracle
 
 
 @pytest.fixture(scope="module")
 def hm():
-    path = arcq_build.build_hostmath()
+    path = arcq_oracle.build_hostmath()
     L = ctypes.CDLL(path)
     vp, i = ctypes.c_void_p, ctypes.c_int
     for n in ("arcq_host_ue4m3", "arcq_host_ue8m0", "arcq_host_e2m1"):

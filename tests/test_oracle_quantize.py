@@ -206,6 +206,39 @@ def test_rmsnorm_quantize(oracle, fmt):
     assert torch.equal(o.view(torch.int16), normed[1].view(torch.int16))
 
 
+def test_rmsnorm_closed_form_every_row(oracle):
+    """The normalisation step at the benchmark's hidden size, every row of a 64 x 4096 case, from scratch
+    in exact arithmetic: the sum of squares of bf16 values as an integer sum (python ints cannot
+    round), mean and 1/sqrt rounded to fp32 where benchmarks/modeling_arc.py:237-242 rounds them, the
+    two bf16 roundings of h and gamma * h.  A dropped term, a wrong divisor (K vs K-1), eps added in
+    the wrong place or a single rounding instead of two each fail it."""
+    from fractions import Fraction
+    M, K, eps = 64, 4096, 1e-5
+    x = make_x(M, K, seed=41, outlier_frac=0.005, outlier_gain=50.0)
+    x[5] = 0
+    x[6] *= 1e-3
+    x[7] *= 300.0
+    g = torch.Generator().manual_seed(42)
+    gamma = (torch.rand(K, generator=g) + 0.5).to(torch.bfloat16)
+    r = oracle.rmsnorm_quantize_x(x, gamma, eps, None, 0, "NVFP4", 1.0, want_normed=True)
+    normed = bits_to_bf16(r["normed"])
+    xd = x.double().numpy()
+    for m in range(M):
+        # every bf16 is an integer multiple of 2^-133: exact integer sum of squares
+        ints = [int(v * 2.0 ** 133) for v in xd[m]]
+        assert all(float(i) * 2.0 ** -133 == v for i, v in zip(ints[:8], xd[m][:8]))
+        mean = Fraction(sum(i * i for i in ints), K) / Fraction(2) ** 266
+        var = np.float32(float(mean))                               # Fraction -> fp64 -> fp32 ...
+        for nb in (np.nextafter(var, np.float32(np.inf)), np.nextafter(var, np.float32(-np.inf))):
+            # ... is the correctly rounded fp32: no neighbour is closer to the exact mean
+            assert abs(Fraction(float(var)) - mean) < abs(Fraction(float(nb)) - mean) or mean == 0
+        a = np.float32(var + np.float32(eps))
+        rstd = np.float32(1.0) / np.sqrt(a, dtype=np.float32)
+        h = (x[m].float() * torch.tensor(rstd)).to(torch.bfloat16)
+        o = (gamma.float() * h.float()).to(torch.bfloat16)
+        assert torch.equal(o.view(torch.int16), normed[m].view(torch.int16)), m
+
+
 @pytest.mark.parametrize("fmt", FMTS)
 def test_matmul_oracle(oracle, fmt):
     M, N, K, S = 9, 11, 256, 64
