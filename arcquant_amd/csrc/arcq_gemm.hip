@@ -1174,8 +1174,80 @@ int matmul_impl(const void *a_codes, const void *a_scales, const void *b_codes, 
   return run_gemm(p, plan, fmt, scratch, st);
 }
 
+// ---------------------------------------------------------------------------------------------
+// arcq_matmul_noalloc: the split-K partial tiles in a fixed array of the code object instead of
+// allocated memory, for callers that cannot allocate.  `scratch` below is the host-side stand-in of
+// that array, not a device address: its address on each device comes from hipGetSymbolAddress, once
+// per device, and only that pointer is handed to kernels.
+// ---------------------------------------------------------------------------------------------
+constexpr size_t kNoAllocScratchBytes = 8u << 20;
+constexpr int kNoAllocMaxDevices = 64;
+
 }  // namespace
 }  // namespace arcq
+
+static __device__ __align__(256) unsigned char scratch[arcq::kNoAllocScratchBytes];
+
+namespace arcq {
+namespace {
+
+// device address of `scratch` on the current device (each device holds its own copy); nullptr + status on failure
+float *noalloc_scratch(int *status) {
+  static std::mutex mu;
+  static float *addr[kNoAllocMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    *status = note_hip_error(e);
+    return nullptr;
+  }
+  if (dev < 0 || dev >= kNoAllocMaxDevices) {
+    *status = ARCQ_ERR_WORKSPACE;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!addr[dev]) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      *status = note_hip_error(e != hipSuccess ? e : hipErrorInvalidSymbol);
+      return nullptr;
+    }
+    addr[dev] = static_cast<float *>(ptr);
+  }
+  return addr[dev];
+}
+
+}  // namespace
+}  // namespace arcq
+
+extern "C" int arcq_matmul_noalloc(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                                   int M, int N, int Kp, int fmt, float alpha, const float *d_alpha_a,
+                                   const float *d_alpha_b, void *c, void *stream) {
+  using namespace arcq;
+  GemmParams p;
+  const int rc = check_gemm_args(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b,
+                                 nullptr, c, &p);
+  if (rc != ARCQ_OK || M == 0 || N == 0) return rc;
+  const GemmPlan plan = plan_gemm(M, N, Kp, fmt, aligned16(a_scales) && aligned16(b_scales));
+  if (plan.scratch_bytes() > kNoAllocScratchBytes) return ARCQ_ERR_WORKSPACE;  // beyond the fixed array: nothing is launched
+  float *ws = nullptr;
+  if (plan.slices > 1) {
+    int status = ARCQ_OK;
+    ws = noalloc_scratch(&status);
+    if (!ws) return status;
+    // every word of the partial tiles that the reduction reads is written by this call's first
+    // launch, so nothing of the previous call's contents has to be cleared
+  }
+  return run_gemm(p, plan, fmt, ws, static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t arcq_matmul_noalloc_limit(void) { return arcq::kNoAllocScratchBytes; }
+
+extern "C" size_t arcq_matmul_scratch_bytes(int M, int N, int Kp, int fmt) {
+  if ((fmt != ARCQ_FMT_NVFP4 && fmt != ARCQ_FMT_MXFP4) || M <= 0 || N <= 0 || Kp < 64 || Kp % 64 != 0) return 0;
+  return arcq::plan_gemm(M, N, Kp, fmt, true).scratch_bytes();
+}
 
 extern "C" int arcq_matmul(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
                            int M, int N, int Kp, int fmt, float alpha, const float *d_alpha_a,

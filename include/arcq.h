@@ -175,6 +175,29 @@ int arcq_matmul_add(const void *a_codes, const void *a_scales, const void *b_cod
                     void *c, void *stream);
 
 /*
+ * arcq_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernel
+ * choice and the same bits as arcq_matmul, but the split-K partial tiles live in a fixed 8 MiB array inside
+ * the library's code object (one copy per GPU, held until the process ends) instead of a stream's scratch
+ * buffer, and the call contains no allocation of any kind.
+ *   - A problem whose plan needs more than arcq_matmul_noalloc_limit() bytes of partial tiles
+ *     (arcq_matmul_scratch_bytes tells, 0 = none needed) is refused with ARCQ_ERR_WORKSPACE and nothing is
+ *     launched: e.g. the 4096 x 14336 down projection at 512 rows (two K slices, 16 MiB).  Every decode batch
+ *     (M <= 64) of the Llama-3-8B shapes fits.
+ *   - All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams,
+ *     two threads) race.  The array keeps the last call's contents; every word a call reads back it has
+ *     written first, so nothing needs clearing.
+ *   - The first call on a device resolves the array's address (hipGetSymbolAddress); make one call, of this
+ *     or any other entry point after loading the library, before a capture.
+ */
+int arcq_matmul_noalloc(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
+                        int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b, void *c,
+                        void *stream);
+size_t arcq_matmul_noalloc_limit(void);
+/* bytes of split-K partial tiles arcq_matmul's plan uses for this problem (0: the plan does not cut K) */
+size_t arcq_matmul_scratch_bytes(int M, int N, int Kp, int fmt);
+
+/*
  * INT4 paged KV cache (the reference's decode-attention path: agemm.init_kv_i4 / append_kv_i4 /
  * batch_decode_i4, kernels/src/bindings.cpp:287-413 -> kernels/src/flashinfer.cu:9-112, with the
  * torch-side quantizer asym_quantize_and_pack_i4, model/kv_cache.py:23-37, fused into the append).
