@@ -41,12 +41,14 @@ void *stream_workspace(int kind, hipStream_t stream, int *status);
 //   ARCQ_GEMM_KERNEL=<WN><WM>   force a GEMM tile (44, 42, 22, 21; 214 / 224 = four-stage ring; 1 = skinny, 0 = direct)
 //   ARCQ_GEMM_SPLITK=<slices>   force split-K for M <= 512 (1 = never split)
 //   ARCQ_QUANT_GRID=<n>         workgroups of the row quantizers
+//   ARCQ_QUANT_KERNEL=<1|2>     1 = never, 2 = always take the wave-per-row quantizer where it has an instance
 //   ARCQ_KV_DECODE_SPLITS=<n>   ranges per sequence of the decode attention
 // Unset (the normal case) every field keeps the value below and the dispatch is the measured one.
 struct Tuning {
   int gemm_kernel = -1;
   int gemm_splitk = 0;
   int quant_grid = 0;
+  int quant_kernel = 0;
   int kv_decode_splits = 0;
 };
 const Tuning &tuning();

@@ -172,6 +172,29 @@ def test_large_shape_properties(agemm, oracle):
         assert e_arc < 0.25 * e_main
 
 
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("M,K,S", [(3072, 4096, 256), (4096, 4096, 64), (3073, 4096, 0), (3500, 4096, 1536),
+                                   (3100, 4096, 4096), (3100, 1024, 128), (3330, 2048, 2048), (3200, 3072, 192),
+                                   (5000, 2048, 64), (9000, 1024, 64)])
+def test_many_rows_unit_scale(agemm, oracle, fmt, M, K, S):
+    """Three thousand rows and more of a hidden size up to 4096 with tensor scale 1: the fused norm takes
+    the wave-per-row kernel there (a wave owns whole rows, one LDS slot per wave refilled in turn); ragged
+    row counts, one to three rows per wave, residual blocks in one or in several of a lane's units
+    (select_num up to K), K = 3072 (mean by division, not by scaling).  The plain quantizer of the same
+    launches is compared as well."""
+    x = recipes.activations(M, K, seed=5000 + M + K + S, outlier_frac=0.005, outlier_gain=50.0)
+    x[M // 3] = 0
+    idx = recipes.reorder_index(x)
+    print(f"many rows {fmt} M={M} K={K} S={S}", flush=True)
+    want = oracle.quantize_x(x, idx, S, fmt, 1.0)
+    q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), S, fmt=fmt)
+    compare("plain", q, sf, want)
+    gam = recipes.gamma(K, seed=8)
+    want = oracle.rmsnorm_quantize_x(x, gam, 1e-5, idx, S, fmt, 1.0)
+    q, sf = agemm.rmsnorm_quantize_x(dev(x), dev(gam), 1e-5, dev(idx), S, fmt=fmt)
+    compare("fused norm", q, sf, want)
+
+
 def test_dequantize_matches_oracle(agemm, oracle):
     x = recipes.activations(12, 512, seed=77)
     idx = recipes.reorder_index(x)
