@@ -72,6 +72,9 @@ def lib() -> ctypes.CDLL:
     L.arcq_check_index.argtypes = [vp, i, vp]
     L.arcq_dequantize.argtypes = [vp, vp, i, i, i, vp, vp]
     L.arcq_stream_probe.argtypes = [vp, vp, sz, sz, vp]
+    L.arcq_stream_probe_variant.argtypes = [vp, vp, sz, sz, i, vp]
+    L.arcq_stream_probe_variant.restype = i
+    L.arcq_stream_probe_variants.restype = i
     for name in ("arcq_reorder_quantize_x", "arcq_reorder_quantize_w", "arcq_rmsnorm_quantize_x", "arcq_matmul",
                  "arcq_check_index", "arcq_dequantize", "arcq_stream_probe", "arcq_swiglu_quantize_x", "arcq_swiglu_absmax",
                  "arcq_kv_append_i4", "arcq_kv_store_i4", "arcq_kv_decode_i4"):

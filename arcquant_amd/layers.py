@@ -329,6 +329,145 @@ class LlamaDecoderLayer(nn.Module):
         return self.mlp(self.post_attention_layernorm(h), residual=h)
 
 
+class SplitQLinear(nn.Module):
+    """Several QLinearLayers over one quantized input, outputs concatenated along the features: q / k / v
+    (or gate / up) kept as the reference keeps them, each with the tensor scale of its own weight
+    (model/qLinearLayer.py:25-28), where the fused layers above have one scale for the stacked weight."""
+
+    def __init__(self, parts):
+        super().__init__()
+        self.parts = nn.ModuleList(parts)
+        self.select_num = parts[0].select_num
+        self.out_features = sum(p.out_features for p in parts)
+
+    @torch.no_grad()
+    def forward(self, x, residual=None):
+        y = torch.cat([p(x) for p in self.parts], dim=-1)
+        return y if residual is None else y + residual
+
+
+class LlamaRMSNorm(nn.Module):
+    """HF's LlamaRMSNorm (benchmarks/modeling_arc.py:237-242): fp32 statistics, the normalised value and
+    its product with the weight each rounded to the input dtype.  model/qLlamaLayer.py:180-197 keeps the
+    model's own norm in front of the quantizer; RMSNormQuant is the fused form."""
+
+    def __init__(self, weight, eps):
+        super().__init__()
+        self.register_buffer("weight", weight.to(torch.bfloat16).contiguous())
+        self.variance_epsilon = float(eps)
+
+    @torch.no_grad()
+    def forward(self, hidden_states):
+        dt = hidden_states.dtype
+        h = hidden_states.to(torch.float32)
+        h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * h.to(dt)
+
+
+CALIBRATION_KEY = "layers.{}.{}.{}.{}"     # model/qLlamaLayer.py:236: layer, block, projection, 'input'
+
+
+def _calibrated(select_nums, reorder_index, i, block, proj, device):
+    key = CALIBRATION_KEY.format(i, block, proj, "input")
+    if key not in select_nums or key not in reorder_index:
+        raise KeyError(f"calibration files hold no entry {key}")
+    return int(select_nums[key]), reorder_index[key].to(device=device, dtype=torch.int16).contiguous()
+
+
+class QLlamaAttention(LlamaAttention):
+    """model/qLlamaLayer.py:207-378 with the reference's constructor arguments: the projections of the
+    original attention block and the two calibration dicts (reorder_indices.py:88-97) keyed
+    'layers.{i}.self_attn.{q,k,v,o}_proj.input'.  q, k and v stay separate QLinearLayers with their own
+    NVFP4 tensor scales, so the weight codes are the reference's; they share one quantized input, taken
+    with q_proj's entry as the reference does (model/qLlamaLayer.py:297)."""
+
+    def __init__(self, q_proj, k_proj, v_proj, o_proj, num_heads, num_kv_heads, select_nums, reorder_index, i,
+                 quant_type="NVFP4"):
+        nn.Module.__init__(self)
+        dev = q_proj.weight.device
+        self.num_heads, self.num_kv_heads = num_heads, num_kv_heads
+        self.head_dim = o_proj.in_features // num_heads
+        self.layer_idx = i
+        parts = []
+        for name, lin in (("q_proj", q_proj), ("k_proj", k_proj), ("v_proj", v_proj)):
+            sel, idx = _calibrated(select_nums, reorder_index, i, "self_attn", name, dev)
+            parts.append(QLinearLayer(lin, sel, idx, quant_type=quant_type))
+        self.qkv_proj = SplitQLinear(parts)
+        self.q_proj, self.k_proj, self.v_proj = parts
+        sel_q, idx_q = _calibrated(select_nums, reorder_index, i, "self_attn", "q_proj", dev)
+        sel_o, idx_o = _calibrated(select_nums, reorder_index, i, "self_attn", "o_proj", dev)
+        for p in parts[1:]:
+            if p.select_num != sel_q:
+                raise ValueError("k_proj / v_proj read q_proj's quantized input: their select_num must equal q_proj's")
+        self.o_proj = QLinearLayer(o_proj, sel_o, idx_o, quant_type=quant_type)
+        self.register_buffer("q_reorder_index", idx_q)
+        self.register_buffer("o_reorder_index", idx_o)
+        self.quant_type = quant_type
+        self._rope = None
+
+
+class QLlamaMLP(LlamaMLP):
+    """model/qLlamaLayer.py:380-443: gate_proj and up_proj separate (own tensor scales), one quantized
+    input taken with up_proj's entry (model/qLlamaLayer.py:429), keys 'layers.{i}.mlp.{gate,up,down}_proj.input'."""
+
+    def __init__(self, gate_proj, up_proj, down_proj, select_nums, reorder_index, i, quant_type="NVFP4"):
+        nn.Module.__init__(self)
+        dev = gate_proj.weight.device
+        self.inter = down_proj.in_features
+        sel_g, idx_g = _calibrated(select_nums, reorder_index, i, "mlp", "gate_proj", dev)
+        sel_u, idx_u = _calibrated(select_nums, reorder_index, i, "mlp", "up_proj", dev)
+        sel_d, idx_d = _calibrated(select_nums, reorder_index, i, "mlp", "down_proj", dev)
+        if sel_g != sel_u:
+            raise ValueError("gate_proj reads up_proj's quantized input: their select_num must be equal")
+        self.gate_proj = QLinearLayer(gate_proj, sel_g, idx_g, quant_type=quant_type)
+        self.up_proj = QLinearLayer(up_proj, sel_u, idx_u, quant_type=quant_type)
+        self.gate_up_proj = SplitQLinear([self.gate_proj, self.up_proj])
+        self.down_proj = QLinearLayer(down_proj, sel_d, idx_d, quant_type=quant_type)
+        self.register_buffer("up_reorder_index", idx_u)
+        self.register_buffer("down_reorder_index", idx_d)
+        self.layer_idx = i
+        self.quant_type = quant_type
+
+
+class QLlamaDecoderLayer(nn.Module):
+    """model/qLlamaLayer.py:88-176 built the reference's way: from a decoder layer's own linears and norm
+    weights plus the calibration dicts.  The norms stay the model's (torch) and every quantizer takes the
+    NVFP4 tensor scale max|x|/2688 of its input, as model/qLlamaLayer.py:73-86 does; fuse_norm=True swaps
+    in the fused RMSNorm -> quantize operator (tensor scale 1: benchmarks/modeling_arc.py:211-227)."""
+
+    def __init__(self, linears, norm_weights, eps, num_heads, num_kv_heads, select_nums, reorder_index, layer_idx,
+                 quant_type="NVFP4", fuse_norm=False):
+        super().__init__()
+        self.self_attn = QLlamaAttention(linears["q_proj"], linears["k_proj"], linears["v_proj"], linears["o_proj"],
+                                         num_heads, num_kv_heads, select_nums, reorder_index, layer_idx, quant_type)
+        self.mlp = QLlamaMLP(linears["gate_proj"], linears["up_proj"], linears["down_proj"], select_nums,
+                             reorder_index, layer_idx, quant_type)
+        self.quant_type = quant_type
+        self.layer_idx = layer_idx
+        if fuse_norm:
+            self.input_layernorm = RMSNormQuant(norm_weights[0], eps, self.self_attn.q_proj.select_num,
+                                                self.self_attn.q_reorder_index, quant_type)
+            self.post_attention_layernorm = RMSNormQuant(norm_weights[1], eps, self.mlp.up_proj.select_num,
+                                                         self.mlp.up_reorder_index, quant_type)
+        else:
+            self.input_layernorm = LlamaRMSNorm(norm_weights[0], eps)
+            self.post_attention_layernorm = LlamaRMSNorm(norm_weights[1], eps)
+        self.fuse_norm = bool(fuse_norm)
+
+    @torch.no_grad()
+    def forward(self, hidden_states, kv_cache=None, past_len=0, layer_idx=None):
+        li = self.layer_idx if layer_idx is None else layer_idx
+        a, m = self.self_attn, self.mlp
+        t = self.input_layernorm(hidden_states)
+        if not self.fuse_norm:
+            t = quantize_tokens(t, a.q_reorder_index, a.q_proj.select_num, self.quant_type)
+        h = a(t, kv_cache, past_len, li, residual=hidden_states)
+        t = self.post_attention_layernorm(h)
+        if not self.fuse_norm:
+            t = quantize_tokens(t, m.up_reorder_index, m.up_proj.select_num, self.quant_type)
+        return m(t, residual=h)
+
+
 class MixtralExpertMLP(nn.Module):
     """model/qMixtralLayer.py:466-543: w2(act(w1 x) * w3 x) on a ragged set of tokens."""
 

@@ -286,6 +286,17 @@ int arcq_dequantize(const void *codes, const void *scales, int rows, int Kp, int
  */
 int arcq_stream_probe(const void *src, void *dst, size_t bytes_in, size_t bytes_out, void *stream);
 
+/*
+ * The same copy with other launch shapes (no counterpart in the reference): variant 0 is
+ * arcq_stream_probe (one 16-byte load in flight per thread); the others keep 2, 4 or 8 independent loads
+ * in flight per thread, use non-temporal loads and stores, run as many workgroups as the chip holds or
+ * exactly one round of threads, or go through LDS-direct loads.  bench.py times all of them on the
+ * headline launch's bytes and reports the fastest as the streaming ceiling of the box.
+ * arcq_stream_probe_variants() is their number; an unknown variant is ARCQ_ERR_SHAPE.
+ */
+int arcq_stream_probe_variant(const void *src, void *dst, size_t bytes_in, size_t bytes_out, int variant, void *stream);
+int arcq_stream_probe_variants(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -246,3 +246,97 @@ def test_chunked_prefill_is_causal(layers):
     second = layer(x[:, 16:].contiguous(), kv, 16)
     assert rel_fro(first, full[:, :16]) < 2e-2
     assert rel_fro(second, full[:, 16:]) < 2e-2
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_decoder_layer_from_calibration_files(layers, fq, oracle, fmt, tmp_path):
+    """The reference's way of building a layer (model/qLlamaLayer.py:88-262): calibration dicts in its
+    file format (reorder_indices.py:88-97), keyed 'layers.{i}.{block}.{proj}.input', loaded from disk and
+    handed to the constructors with the layer's own nn.Linear modules.  q / k / v / gate / up stay
+    separate, each with the NVFP4 tensor scale of its own weight: their weight codes and scale bytes are
+    compared bit for bit with the oracle's per-projection quantizer, the layer output with the
+    fake-quant flow on the CPU."""
+    from arcquant_amd import calibration as cal
+    hidden, inter, nh, nkv, eps, li = 256, 512, 4, 2, 1e-5, 3
+    bsz, q_len = 2, 24
+    d = hidden // nh
+    g = torch.Generator().manual_seed(41)
+    shapes = {"q_proj": (nh * d, hidden), "k_proj": (nkv * d, hidden), "v_proj": (nkv * d, hidden),
+              "o_proj": (hidden, hidden), "gate_proj": (inter, hidden), "up_proj": (inter, hidden),
+              "down_proj": (hidden, inter)}
+    gain = {"q_proj": 1.0, "k_proj": 3.0, "v_proj": 0.5, "o_proj": 1.0, "gate_proj": 2.0, "up_proj": 0.7, "down_proj": 1.0}
+    W = {k: (torch.randn(*s, generator=g) * 0.02 * gain[k]).to(torch.bfloat16) for k, s in shapes.items()}
+    g1 = (torch.rand(hidden, generator=g) + 0.5).to(torch.bfloat16)
+    g2 = (torch.rand(hidden, generator=g) + 0.5).to(torch.bfloat16)
+    x = torch.randn(bsz, q_len, hidden, generator=g)
+    x[..., 7] *= 20.0
+    x = x.to(torch.bfloat16)
+
+    # calibration statistics: per-channel max |activation| of each linear's input on a calibration batch
+    # (utilize.py:39-45); here random statistics per input, written and read back in the reference's format
+    stat = {"attn": torch.rand(hidden, generator=g), "o": torch.rand(hidden, generator=g),
+            "mlp": torch.rand(hidden, generator=g), "down": torch.rand(inter, generator=g)}
+    block_of = {"q_proj": ("self_attn", "attn", 64), "k_proj": ("self_attn", "attn", 64), "v_proj": ("self_attn", "attn", 64),
+                "o_proj": ("self_attn", "o", 128), "gate_proj": ("mlp", "mlp", 64), "up_proj": ("mlp", "mlp", 64),
+                "down_proj": ("mlp", "down", 192)}
+    ri, sn = {}, {}
+    for proj, (block, st, sel) in block_of.items():
+        key = cal.NAME_TEMPLATE.format(li, block, proj)
+        ri[key] = cal.reorder_index_from_stat(stat[st])
+        sn[key] = sel
+    cal.save_reorder_index(tmp_path / "reorder_index.pt", ri)
+    cal.save_select_num(tmp_path / "select_num.pt", sn)
+    ri, sn = cal.load_reorder_index(tmp_path / "reorder_index.pt"), cal.load_select_num(tmp_path / "select_num.pt")
+
+    lin = {}
+    for k, (n_out, n_in) in shapes.items():
+        lin[k] = nn.Linear(n_in, n_out, bias=False, device="cuda", dtype=torch.bfloat16)
+        lin[k].weight.data.copy_(W[k])
+    print(f"calibrated decoder layer {fmt}", flush=True)
+    layer = layers.QLlamaDecoderLayer(lin, (g1.cuda(), g2.cuda()), eps, nh, nkv, sn, ri, li, quant_type=fmt)
+    with pytest.raises(KeyError):
+        layers.QLlamaDecoderLayer(lin, (g1.cuda(), g2.cuda()), eps, nh, nkv, sn, ri, li + 1, quant_type=fmt)
+
+    # weight codes / scales of every projection = the oracle's quantizer with that projection's own tensor scale
+    mods = {"q_proj": layer.self_attn.q_proj, "k_proj": layer.self_attn.k_proj, "v_proj": layer.self_attn.v_proj,
+            "o_proj": layer.self_attn.o_proj, "gate_proj": layer.mlp.gate_proj, "up_proj": layer.mlp.up_proj,
+            "down_proj": layer.mlp.down_proj}
+    idx_of = {}
+    for proj, (block, st, sel) in block_of.items():
+        idx = ri[cal.NAME_TEMPLATE.format(li, block, proj)].to(torch.int16)
+        idx_of[proj] = (idx, sel)
+        gw = recipes.tensor_scale(W[proj], fmt)
+        want = oracle.quantize_w(W[proj], idx, sel, fmt, gw)
+        m = mods[proj]
+        assert (m.W.cpu().numpy() == want["codes"]).all(), proj
+        assert (m.scale_w.cpu().numpy().reshape(want["scales"].shape) == want["scales"]).all(), proj
+        assert float(m.scale) == pytest.approx(gw, rel=1e-7)
+    if fmt == "NVFP4":
+        assert len({float(mods[p].scale) for p in ("q_proj", "k_proj", "v_proj")}) == 3
+
+    y = layer(x.cuda())
+    assert y.shape == x.shape
+
+    def lin_ref(t, proj):
+        idx, sel = idx_of[proj]
+        return ref_linear(fq, t, W[proj], idx, sel, fmt)
+
+    x2 = x.view(-1, hidden)
+    n1 = fq.hf_rmsnorm(x2, g1, eps)
+    qkv = torch.cat([lin_ref(n1, p) for p in ("q_proj", "k_proj", "v_proj")], dim=1)
+    q = qkv[:, :nh * d].view(bsz, q_len, nh, d).transpose(1, 2)
+    k = qkv[:, nh * d:(nh + nkv) * d].view(bsz, q_len, nkv, d).transpose(1, 2)
+    v = qkv[:, (nh + nkv) * d:].view(bsz, q_len, nkv, d).transpose(1, 2)
+    q, k = layers.rotary_pos_emb(q, k, 0)
+    k, v = k.repeat_interleave(nh // nkv, 1), v.repeat_interleave(nh // nkv, 1)
+    o = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True).to(torch.bfloat16)
+    h = x2 + lin_ref(o.transpose(1, 2).reshape(bsz * q_len, hidden), "o_proj")
+    n2 = fq.hf_rmsnorm(h, g2, eps)
+    t = F.silu(lin_ref(n2, "gate_proj")) * lin_ref(n2, "up_proj")
+    want = h + lin_ref(t, "down_proj")
+    assert rel_fro(y.view(-1, hidden), want) < 2e-2       # as test_decoder_layer_matches_fake_quant_flow
+
+    # the fused norm -> quantize form of the same layer (tensor scale 1) stays within quantization noise of it
+    fused = layers.QLlamaDecoderLayer(lin, (g1.cuda(), g2.cuda()), eps, nh, nkv, sn, ri, li, quant_type=fmt,
+                                      fuse_norm=True)
+    assert rel_fro(fused(x.cuda()), y) < 0.1
