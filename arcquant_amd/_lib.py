@@ -69,6 +69,15 @@ def lib() -> ctypes.CDLL:
         L.arcq_matmul_noalloc_limit.restype = sz
         L.arcq_matmul_scratch_bytes.argtypes = [i, i, i, i]
         L.arcq_matmul_scratch_bytes.restype = sz
+    L.arcq_grouped_reorder_quantize_x.argtypes = [vp, i, i, vp, i, vp, i, i, vp, vp, vp, vp]
+    L.arcq_grouped_swiglu_quantize_x.argtypes = [vp, vp, i, i, i, vp, i, vp, i, i, vp, vp, vp, vp]
+    L.arcq_grouped_tensor_scale.argtypes = [vp, vp, i, i, i, vp, i, f, vp, vp]
+    L.arcq_grouped_matmul.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, f, vp, vp, vp, vp, vp]
+    L.arcq_moe_combine.argtypes = [vp, vp, vp, i, i, i, i, vp, vp]
+    L.arcq_moe_combine.restype = i
+    for name in ("arcq_grouped_reorder_quantize_x", "arcq_grouped_swiglu_quantize_x", "arcq_grouped_tensor_scale",
+                 "arcq_grouped_matmul"):
+        getattr(L, name).restype = i
     L.arcq_check_index.argtypes = [vp, i, vp]
     L.arcq_dequantize.argtypes = [vp, vp, i, i, i, vp, vp]
     L.arcq_stream_probe.argtypes = [vp, vp, sz, sz, vp]

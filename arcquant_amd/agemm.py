@@ -32,7 +32,8 @@ from ._lib import FORMATS, ArcqError  # noqa: F401
 
 __all__ = ["matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "init_kv_i4", "append_kv_i4",
            "batch_decode_i4", "swiglu_quantize_x", "tensor_scale", "prepare_stream", "dequantize", "check_index",
-           "unpack_codes", "scale_values"]
+           "unpack_codes", "scale_values", "grouped_tensor_scale", "grouped_reorder_quantize_x",
+           "grouped_swiglu_quantize_x", "grouped_matmul", "moe_combine"]
 
 
 def _fmt_id(fmt) -> int:
@@ -241,6 +242,156 @@ def matmul(A, B, SFA, SFB, scale, *, fmt=None, residual=None):
     _lib.check(rc, "arcq_matmul")
     del ka, kb
     return C
+
+
+# ------------------------------------------------------------------------------------------
+# grouped operators for mixture-of-experts blocks: rows sorted by expert, `seg` int32 [E+1] row
+# offsets on the device, one launch per step for all experts and no host read-back
+# (model/qMixtralLayer.py:458-471 walks the experts in Python instead)
+# ------------------------------------------------------------------------------------------
+
+def _seg(seg, device):
+    _require(seg, "seg", torch.int32, 1)
+    if seg.device != device or seg.numel() < 2:
+        raise RuntimeError("seg must be an int32 tensor [experts + 1] on the operands' device")
+    return seg.numel() - 1
+
+
+def _rows_2d(t, name):
+    if not isinstance(t, torch.Tensor) or t.dtype != torch.bfloat16 or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1:
+        raise RuntimeError(f"{name} must be a 2-D bf16 CUDA tensor with unit stride along its last dimension")
+    M, K = t.shape
+    ld = t.stride(0) if M > 1 else K
+    if ld % 8 or t.data_ptr() % 16:
+        raise RuntimeError(f"{name}: row stride {ld} / alignment not supported")
+    return M, K, ld
+
+
+def grouped_tensor_scale(x, seg, divisor=2688.0, *, up=None):
+    """NVFP4 tensor scales max|x_e| / divisor of each expert's rows of x (bf16 [M, K]) as fp32 [E] on the
+    device (1 for an expert without rows); with `up`, of act_fn(x) * up (x = gate)."""
+    M, K, ld = _rows_2d(x, "x")
+    E = _seg(seg, x.device)
+    if up is not None:
+        if _rows_2d(up, "up") != (M, K, ld):
+            raise RuntimeError("gate and up must have the same shape and row stride")
+    out = torch.empty(E, dtype=torch.float32, device=x.device)
+    with _on_device(x):
+        rc = _lib.lib().arcq_grouped_tensor_scale(x.data_ptr(), None if up is None else up.data_ptr(), ld, M, K,
+                                                  seg.data_ptr(), E, float(divisor), out.data_ptr(), _stream(x))
+    _lib.check(rc, "arcq_grouped_tensor_scale")
+    return out
+
+
+def _grouped_quantize(gate, up, seg, reorder_index, KE, fmt, global_scales):
+    f = _fmt_id(fmt)
+    M, K, ld = _rows_2d(gate, "x" if up is None else "gate")
+    E = _seg(seg, gate.device)
+    _require(reorder_index, "reorder_index", torch.int16, 2)
+    KE = int(KE)
+    G = _lib.GROUP_SIZE[f]
+    if tuple(reorder_index.shape) != (E, K) or reorder_index.device != gate.device:
+        raise RuntimeError(f"reorder_index must be int16 [{E}, {K}] on the operands' device")
+    if K % 32 or K < 32 or K > 16384 or KE < 0 or KE > K or KE % G:
+        raise RuntimeError(f"Value error in grouped quantizer: K={K}, KE={KE} not supported for {fmt}")
+    if global_scales is not None:
+        _require(global_scales, "global_scales", torch.float32, 1)
+        if global_scales.numel() != E or global_scales.device != gate.device:
+            raise RuntimeError(f"global_scales must be fp32 [{E}] on the operands' device")
+    QX = torch.empty((M, (K + KE) // 2), dtype=torch.uint8, device=gate.device)
+    SFX = torch.empty((M * ((K + KE) // G),), dtype=torch.uint8, device=gate.device)
+    L = _lib.lib()
+    d_gs = None if global_scales is None else global_scales.data_ptr()
+    with _on_device(gate):
+        if up is None:
+            if ld != K:
+                raise RuntimeError("x must be contiguous")
+            rc = L.arcq_grouped_reorder_quantize_x(gate.data_ptr(), M, K, seg.data_ptr(), E, reorder_index.data_ptr(), KE,
+                                                   f, d_gs, QX.data_ptr(), SFX.data_ptr(), _stream(gate))
+        else:
+            rc = L.arcq_grouped_swiglu_quantize_x(gate.data_ptr(), up.data_ptr(), ld, M, K, seg.data_ptr(), E,
+                                                  reorder_index.data_ptr(), KE, f, d_gs, QX.data_ptr(), SFX.data_ptr(),
+                                                  _stream(gate))
+    _lib.check(rc, "grouped quantizer")
+    return QX, SFX
+
+
+def grouped_reorder_quantize_x(X, seg, reorder_index, KE, *, fmt="NVFP4", global_scales=None):
+    """reorder_quantize_x over tokens sorted by expert: row r in seg[e] .. seg[e+1]-1 is quantized with
+    reorder_index[e] and tensor scale global_scales[e] (None: 1).  X bf16 [M, K] contiguous."""
+    return _grouped_quantize(X, None, seg, reorder_index, KE, fmt, global_scales)
+
+
+def grouped_swiglu_quantize_x(gate, up, seg, reorder_index, KE, *, fmt="NVFP4", global_scales=None):
+    """swiglu_quantize_x over tokens sorted by expert; global_scales: fp32 [E], None, or "absmax" (the
+    per-expert NVFP4 scales are computed on the device first and returned as a third value)."""
+    if isinstance(global_scales, str):
+        if global_scales != "absmax":
+            raise RuntimeError("global_scales must be a tensor, None or 'absmax'")
+        gs = grouped_tensor_scale(gate, seg, 2688.0, up=up)
+        return _grouped_quantize(gate, up, seg, reorder_index, KE, fmt, gs) + (gs,)
+    if _rows_2d(up, "up") != _rows_2d(gate, "gate"):
+        raise RuntimeError("gate and up must have the same shape and row stride")
+    return _grouped_quantize(gate, up, seg, reorder_index, KE, fmt, global_scales)
+
+
+def grouped_matmul(A, B, SFA, SFB, seg, scale_a=None, scale_b=None, *, fmt=None, residual=None):
+    """Rows seg[e] .. seg[e+1]-1 of bf16 [M, N] = scale_a[e] * scale_b[e] * dq(A rows) @ dq(B[e])^T.
+    A u8 [M, K'/2]; B u8 [E, N, K'/2], SFB u8 [E * N * K'/G]: the experts' quantized weights stacked;
+    scale_a / scale_b fp32 [E] on the device or None."""
+    _require(A, "A", torch.uint8, 2)
+    _require(B, "B", torch.uint8, 3)
+    _require(SFA, "SFA", torch.uint8)
+    _require(SFB, "SFB", torch.uint8)
+    E = _seg(seg, A.device)
+    if B.shape[0] != E or A.shape[1] != B.shape[2]:
+        raise RuntimeError(f"B must be [{E}, N, {A.shape[1]}]")
+    f = _infer_fmt(A, SFA, fmt)
+    M, N, Kp = A.shape[0], B.shape[1], 2 * A.shape[1]
+    G = _lib.GROUP_SIZE[f]
+    if SFA.numel() != M * (Kp // G) or SFB.numel() != E * N * (Kp // G):
+        raise RuntimeError("scale buffers do not match the code buffers")
+    if Kp % 128 or Kp < 512:
+        raise RuntimeError(f"Value error in grouped_matmul: K'={Kp} must be a multiple of 128, at least 512")
+    ptrs = []
+    for t, name in ((scale_a, "scale_a"), (scale_b, "scale_b")):
+        if t is None:
+            ptrs.append(None)
+            continue
+        _require(t, name, torch.float32, 1)
+        if t.numel() != E or t.device != A.device:
+            raise RuntimeError(f"{name} must be fp32 [{E}] on A's device")
+        ptrs.append(t.data_ptr())
+    if residual is not None:
+        _require(residual, "residual", torch.bfloat16, 2)
+        if tuple(residual.shape) != (M, N) or residual.device != A.device:
+            raise RuntimeError(f"residual must be bf16 [{M}, {N}] on A's device")
+    C = torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
+    with _on_device(A):
+        rc = _lib.lib().arcq_grouped_matmul(A.data_ptr(), SFA.data_ptr(), B.data_ptr(), SFB.data_ptr(), seg.data_ptr(), E,
+                                            M, N, Kp, f, 1.0, ptrs[0], ptrs[1],
+                                            None if residual is None else residual.data_ptr(), C.data_ptr(), _stream(A))
+    _lib.check(rc, "arcq_grouped_matmul")
+    return C
+
+
+def moe_combine(y, position, weight, tokens, top_k):
+    """out[t] = sum over token t's experts (ascending expert number) of bf16(y[row] * weight[row]), partial sums
+    rounded to bf16: the weighting and index_add_ of model/qMixtralLayer.py:466-471 in one launch.
+    y bf16 [pairs, H] in expert-sorted order, position int64 [tokens * top_k] (row of y per (token, slot)),
+    weight bf16 [pairs] in sorted order."""
+    _require(y, "y", torch.bfloat16, 2)
+    _require(position, "position", torch.int64, 1)
+    _require(weight, "weight", torch.bfloat16, 1)
+    pairs, H = y.shape
+    if position.numel() != tokens * top_k or weight.numel() != pairs or H % 8 or not 1 <= top_k <= 8:
+        raise RuntimeError(f"Value error in moe_combine: pairs={pairs}, H={H}, tokens={tokens}, top_k={top_k}")
+    out = torch.empty((tokens, H), dtype=torch.bfloat16, device=y.device)
+    with _on_device(y):
+        rc = _lib.lib().arcq_moe_combine(y.data_ptr(), position.data_ptr(), weight.data_ptr(), tokens, H, top_k, pairs,
+                                         out.data_ptr(), _stream(y))
+    _lib.check(rc, "arcq_moe_combine")
+    return out
 
 
 def prepare_stream(device=None) -> None:

@@ -15,7 +15,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-HIP_SOURCES = ["arcq_common.hip", "arcq_quantize.hip", "arcq_gemm.hip", "arcq_kvcache.hip"]
+HIP_SOURCES = ["arcq_common.hip", "arcq_quantize.hip", "arcq_gemm.hip", "arcq_kvcache.hip", "arcq_moe.hip"]
 HIP_LIB = os.path.join(CSRC, "libarcq_hip.so")
 
 HIPCC_FLAGS = [

@@ -41,7 +41,47 @@ struct GemmParams {
   // optional residual, bf16 [M,N]: C = bf16(bf16(alpha * acc) + residual), what a bf16 add of the
   // rounded GEMM output and the residual gives
   const uint16_t *residual = nullptr;
+  // grouped GEMM (tiled kernels): rows seg[e] .. seg[e+1]-1 of A and C belong to segment e, whose weights
+  // start seg_b_codes / seg_b_scales bytes after those of segment e-1; d_alpha_a / d_alpha_b are arrays
+  // indexed by segment.  A workgroup rewrites its copy of these parameters to its segment's sub-problem.
+  const int *seg = nullptr;
+  int n_seg = 0;
+  size_t seg_b_codes = 0, seg_b_scales = 0;
 };
+
+// Grouped launches: maps the workgroup to (segment, tile) and turns p into that segment's problem (M = its
+// rows, operand pointers moved to its first row and its weights).  lin: tile number inside the segment, in
+// the order the ungrouped kernels use.  The launch holds an upper bound of the tile count; workgroups
+// beyond the real count return false.  G: elements per scale byte.
+template <int BM, int BN, int G>
+__device__ __forceinline__ bool enter_segment(GemmParams &p, int &lin) {
+  const int tiles_n = (p.N + BN - 1) / BN;
+  const int per_xcd = gridDim.x >> 3;  // the grid is a multiple of 8: contiguous runs of tiles per XCD
+  lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int rows = p.M;
+  int beg = min(max(p.seg[0], 0), rows);
+  for (int e = 0; e < p.n_seg; ++e) {
+    const int end = min(max(p.seg[e + 1], beg), rows);  // offsets that do not grow or leave the tensor: empty segments
+    const int cnt = end - beg;
+    const int t = ((cnt + BM - 1) / BM) * tiles_n;
+    if (lin < t) {
+      const size_t kbytes = p.Kp >> 1, ksc = p.Kp / G;
+      p.a_codes += (size_t)beg * kbytes;
+      p.a_scales += (size_t)beg * ksc;
+      p.c += (size_t)beg * p.N;
+      if (p.residual) p.residual += (size_t)beg * p.N;
+      p.b_codes += (size_t)e * p.seg_b_codes;
+      p.b_scales += (size_t)e * p.seg_b_scales;
+      if (p.d_alpha_a) p.d_alpha_a += e;
+      if (p.d_alpha_b) p.d_alpha_b += e;
+      p.M = cnt;
+      return true;
+    }
+    lin -= t;
+    beg = end;
+  }
+  return false;
+}
 
 // two bf16 pairs + two bf16 pairs, each sum rounded to bf16
 __device__ __forceinline__ uint32_t add_bf16_pair(uint32_t a, uint32_t b) {
@@ -359,11 +399,16 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
 
   // tile of this workgroup: consecutive workgroup ids go to different XCDs (8 of them, each with
   // its own L2), so hand each XCD a contiguous run of tiles that walk down M for a fixed weight tile
-  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-  const int total = tiles_m * tiles_n;
-  const int per_xcd = (total + 7) >> 3;
-  const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (lin >= total) return;
+  int lin;
+  if (p.seg) {
+    if (!enter_segment<BM, BN, 32>(p, lin)) return;
+  } else {
+    const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+    const int per_xcd = (total + 7) >> 3;
+    lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (lin >= total) return;
+  }
+  const int tiles_m = (p.M + BM - 1) / BM;
   const int n_base = (lin / tiles_m) * BN, m_base = (lin % tiles_m) * BM;
 
   const int nk = (p.Kp + 255) >> 8;
@@ -586,11 +631,16 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kbytes = p.Kp >> 1, ksc = p.Kp >> 4;
 
-  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-  const int total = tiles_m * tiles_n;
-  const int per_xcd = (total + 7) >> 3;
-  const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (lin >= total) return;
+  int lin;
+  if (p.seg) {
+    if (!enter_segment<BM, BN, 16>(p, lin)) return;
+  } else {
+    const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+    const int per_xcd = (total + 7) >> 3;
+    lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (lin >= total) return;
+  }
+  const int tiles_m = (p.M + BM - 1) / BM;
   const int n_base = (lin / tiles_m) * BN, m_base = (lin % tiles_m) * BM;
 
   const int nk = (p.Kp + 255) >> 8;
@@ -960,7 +1010,8 @@ int launch_skinny_for(const GemmParams &p, hipStream_t st) {
 template <int WN, int WM>
 int launch_nvfp4_tiled(const GemmParams &p, hipStream_t st) {
   constexpr int BN = 64 * WN, BM = 64 * WM;
-  const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  // grouped: every segment may end in one partial tile of rows
+  const int total = ((p.M + BM - 1) / BM + (p.seg ? p.n_seg : 0)) * ((p.N + BN - 1) / BN);
   const int grid = ((total + 7) / 8) * 8;
   hipLaunchKernelGGL((gemm_nvfp4_tiled<WN, WM>), dim3(grid, p.k_slices), dim3(256), 0, st, p);
   ARCQ_HIP_TRY(hipGetLastError());
@@ -970,7 +1021,8 @@ int launch_nvfp4_tiled(const GemmParams &p, hipStream_t st) {
 template <int WN, int WM, int NS = 2>
 int launch_mxfp4_tiled(const GemmParams &p, hipStream_t st) {
   constexpr int BN = 64 * WN, BM = 64 * WM;
-  const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  // grouped: every segment may end in one partial tile of rows
+  const int total = ((p.M + BM - 1) / BM + (p.seg ? p.n_seg : 0)) * ((p.N + BN - 1) / BN);
   const int grid = ((total + 7) / 8) * 8;  // whole groups of 8 so that the XCD split covers every tile
   hipLaunchKernelGGL((gemm_mxfp4_tiled<WN, WM, NS>), dim3(grid, p.k_slices), dim3(256), 0, st, p);
   ARCQ_HIP_TRY(hipGetLastError());
@@ -1263,4 +1315,33 @@ extern "C" int arcq_matmul_add(const void *a_codes, const void *a_scales, const 
   if (!arcq::aligned16(residual)) return ARCQ_ERR_ALIGN;
   return arcq::matmul_impl(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b, residual, c,
                            stream);
+}
+
+extern "C" int arcq_grouped_matmul(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                                   const int *seg_offsets, int n_seg, int M, int N, int Kp, int fmt, float alpha,
+                                   const float *d_alpha_a, const float *d_alpha_b, const void *residual, void *c,
+                                   void *stream) {
+  using namespace arcq;
+  GemmParams p;
+  const int rc = check_gemm_args(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b,
+                                 residual, c, &p);
+  if (rc != ARCQ_OK || M == 0 || N == 0) return rc;
+  if (n_seg < 1 || Kp % 128 != 0 || Kp < 512) return ARCQ_ERR_SHAPE;  // the tiled kernels' shapes only
+  if (!seg_offsets) return ARCQ_ERR_NULL;
+  if (!aligned16(a_scales) || !aligned16(b_scales) || (residual && !aligned16(residual))) return ARCQ_ERR_ALIGN;
+  const int G = fmt == ARCQ_FMT_NVFP4 ? 16 : 32;
+  p.seg = seg_offsets;
+  p.n_seg = n_seg;
+  p.seg_b_codes = (size_t)N * (Kp >> 1);
+  p.seg_b_scales = (size_t)N * (Kp / G);
+  // Tile from the rows an average segment holds (the real counts live on the device).  The larger tiles are
+  // faster per flop, but every segment ends in a partly empty tile of rows and skewed routing leaves some
+  // segments far below the average: on 8192 rows over 8 segments of 195..3120 rows the 128x128 tile beat
+  // 256x128 and 256x256 for both formats (two GEMMs: 1.82 / 1.99 / 1.93 ms MXFP4, 3.80 / 3.87 / 3.87 NVFP4).
+  const int avg = M / n_seg;
+  GemmPlan plan;
+  const int force = tuning().gemm_kernel;
+  plan.kernel = avg >= 2048 ? 44 : (avg >= 96 ? 22 : 21);
+  if (force == 44 || force == 42 || force == 22 || force == 21) plan.kernel = force;
+  return run_gemm(p, plan, fmt, nullptr, static_cast<hipStream_t>(stream));
 }

@@ -40,6 +40,10 @@ struct QuantParams {
   float eps;
   int rows, K, S;
   double inv_k;           // 1/K (MODE_NORM)
+  // grouped launches (rows sorted by segment, e.g. tokens by expert): rows seg[e] .. seg[e+1]-1 take
+  // reorder_index row e of idx [n_seg, K] and tensor scale d_gscale[e]
+  const int *seg = nullptr;
+  int n_seg = 0;
 };
 
 // Block scale from the block's amax: t = amax/6 (quantize.py:155 / :184), then the format's rounding.
@@ -397,7 +401,7 @@ __device__ __forceinline__ uint32_t swiglu_pair(uint32_t gw, uint32_t uw) {
   return pack_bf16_rne(dot2_bf16(a, uw & 0xffffu), dot2_bf16(a, uw & 0xffff0000u));
 }
 
-template <int FMT, int MODE, bool SCALED>
+template <int FMT, int MODE, bool SCALED, bool GROUPED = false>
 __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p) {
   extern __shared__ uint4 smem[];
   constexpr int G = FMT == ARCQ_FMT_NVFP4 ? 16 : 32;
@@ -418,12 +422,14 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
   // SCALED: x32 = x / g (quantize.py:330) as q + (x - g*q)*rg with q = x*rg, rg = RN(1/g): the
   // correctly rounded quotient for every bf16 x (checked exhaustively on the host).  A tensor scale
   // outside 2^-60..2^60 in magnitude sends every unit through unit_exact.
-  const float g = SCALED ? (p.d_gscale ? *p.d_gscale : p.gscale) : 1.0f;
-  const float rg = SCALED ? 1.0f / g : 1.0f;
-  const bool g_odd = SCALED && !(fabsf(g) >= 0x1p-60f && fabsf(g) <= 0x1p+60f);
+  // GROUPED: the scale (and the channel order below) belong to the segment of the row and are
+  // replaced when the workgroup's rows enter another segment
+  float g = SCALED ? (p.d_gscale ? *p.d_gscale : p.gscale) : 1.0f;
+  float rg = SCALED ? 1.0f / g : 1.0f;
+  bool g_odd = SCALED && !(fabsf(g) >= 0x1p-60f && fabsf(g) <= 0x1p+60f);
   // a power-of-two tensor scale leaves bf16 operands bf16-valued: the coarse encode applies (and
   // such operands sit on the grid's ties far too often for the two-sided test to pay)
-  const bool coarse = !SCALED || (f2u(g) & 0x7fffffu) == 0u;
+  bool coarse = !SCALED || (f2u(g) & 0x7fffffu) == 0u;
   // var + eps >= eps: with eps comfortably normal the square root needs no range scaling
   const bool eps_normal = p.eps >= 0x1p-90f;
 
@@ -444,16 +450,20 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
   // channel-only state, loaded once
   uint32_t addr[16];
   uint32_t glo[8], ghi[8];
-  {
+  auto gather_addresses = [&](const int16_t *idx) {
     const uint32_t base = (uint32_t)reinterpret_cast<uintptr_t>(row);
     uint4 i0 = make_uint4(0, 0, 0, 0), i1 = i0;
     if (active) {
-      i0 = reinterpret_cast<const uint4 *>(p.idx)[2 * tid];
-      i1 = reinterpret_cast<const uint4 *>(p.idx)[2 * tid + 1];
+      i0 = reinterpret_cast<const uint4 *>(idx)[2 * tid];
+      i1 = reinterpret_cast<const uint4 *>(idx)[2 * tid + 1];
     }
     const uint32_t iw[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
 #pragma unroll
     for (int i = 0; i < 16; ++i) addr[i] = base + 2u * ((iw[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+  };
+  if (!GROUPED) gather_addresses(p.idx);
+  int seg_cur = -1, seg_end = 0;  // GROUPED: rows below seg_end belong to segment seg_cur (or to an earlier one)
+  {
     if (MODE == MODE_NORM) {
       uint4 g0 = make_uint4(0, 0, 0, 0), g1 = g0;
       if (active) {
@@ -473,6 +483,20 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
   for (int i = 0; i < 16; ++i) yv[i] = 0u;  // low halves stay zero: only d16_hi loads write these
 
   for (; r < p.rows; r += gridDim.x) {
+    if (GROUPED && r >= seg_end) {  // workgroup-uniform: the rows are sorted, so this happens once per segment at most
+      while (seg_cur + 1 < p.n_seg && r >= seg_end) {
+        ++seg_cur;
+        seg_end = p.seg[seg_cur + 1];
+      }
+      if (r >= seg_end) break;  // rows behind the last segment belong to nobody
+      gather_addresses(p.idx + (size_t)seg_cur * K);
+      if (SCALED) {
+        g = p.d_gscale[seg_cur];
+        rg = 1.0f / g;
+        g_odd = !(fabsf(g) >= 0x1p-60f && fabsf(g) <= 0x1p+60f);
+        coarse = (f2u(g) & 0x7fffffu) == 0u;
+      }
+    }
     uint4 n0, n1, un0, un1;  // left undefined past the last row: nothing reads them then
     if (r + (int)gridDim.x < p.rows && active) {  // prefetch the next row of this workgroup
       const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)(r + gridDim.x) * ldx);
@@ -947,7 +971,89 @@ __global__ __launch_bounds__(256) void tensor_scale_kernel(const uint16_t *x, co
   atomicExch(ws + 1, 0u);
 }
 
-template <int FMT, int MODE, bool SCALED>
+// Per-segment maxima for grouped launches (rows sorted by segment): max |x|, or max |act_fn(gate) * up|,
+// over the rows of each segment, accumulated as the bits of a non-negative float in bits[segment] (zeroed
+// by the caller's launch in front).  A workgroup walks rows with stride gridDim and flushes its running
+// maximum with one atomicMax when its rows enter another segment, and at the end.
+template <bool SWIGLU>
+__global__ __launch_bounds__(256) void grouped_absmax_kernel(const uint16_t *x, const uint16_t *up, size_t ld, int rows,
+                                                             int K, const int *seg, int n_seg, uint32_t *bits) {
+  __shared__ uint32_t wave_max[4];
+  const int cpr = K >> 3;  // 16-byte chunks per row
+  int seg_cur = -1, seg_end = 0;
+  uint32_t m = 0u;
+  auto flush = [&]() {  // workgroup-uniform
+    if (seg_cur < 0) return;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t v = (uint32_t)__shfl_xor((int)m, o);
+      m = v > m ? v : m;
+    }
+    __syncthreads();  // the previous flush's readers are done with wave_max
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int w = 1; w < 4; ++w) m = wave_max[w] > m ? wave_max[w] : m;
+      if (m) atomicMax(bits + seg_cur, m);
+    }
+    m = 0u;
+  };
+  for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+    if (r >= seg_end) {
+      flush();
+      while (seg_cur + 1 < n_seg && r >= seg_end) {
+        ++seg_cur;
+        seg_end = seg[seg_cur + 1];
+      }
+      if (r >= seg_end) {  // behind the last segment
+        seg_cur = -1;
+        break;
+      }
+    }
+    // four rows of the workgroup at a time while they stay inside the segment: all their loads are issued
+    // before the first maximum is taken (a row of a few thousand channels is only two loads per thread)
+    const int nr = (!SWIGLU && (long)r + 3L * gridDim.x < (long)min(seg_end, rows)) ? 4 : 1;
+    for (int c = threadIdx.x; c < cpr; c += 256) {
+      uint4 gq[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (j < nr) gq[j] = *reinterpret_cast<const uint4 *>(x + (size_t)(r + j * (int)gridDim.x) * ld + 8 * c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (j >= nr) break;
+        uint32_t t[4] = {gq[j].x, gq[j].y, gq[j].z, gq[j].w};
+        if (SWIGLU) {
+          const uint4 uq = *reinterpret_cast<const uint4 *>(up + (size_t)r * ld + 8 * c);
+          t[0] = swiglu_pair(gq[j].x, uq.x), t[1] = swiglu_pair(gq[j].y, uq.y);
+          t[2] = swiglu_pair(gq[j].z, uq.z), t[3] = swiglu_pair(gq[j].w, uq.w);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t lo = (t[i] << 16) & 0x7fffffffu, hi = t[i] & 0x7fff0000u;
+          m = lo > m ? lo : m;
+          m = hi > m ? hi : m;
+        }
+      }
+    }
+    r += (nr - 1) * (int)gridDim.x;
+  }
+  flush();
+}
+
+__global__ void zero_words_kernel(uint32_t *w, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) w[i] = 0u;
+}
+
+// bits of the maxima -> tensor scales max / divisor in place (IEEE division; an all-zero or empty segment gets 1)
+__global__ void grouped_scale_finish_kernel(uint32_t *bits, int n, float divisor) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float scale = u2f(bits[i]) / divisor;
+  reinterpret_cast<float *>(bits)[i] = scale == 0.0f ? 1.0f : scale;
+}
+
+template <int FMT, int MODE, bool SCALED, bool GROUPED = false>
 int launch_quantize_unit(const QuantParams &p, hipStream_t stream) {
   const int threads = (((p.K >> 4) + 63) / 64) * 64;
   const size_t lds = (size_t)p.K * 2 + 16 * sizeof(double);
@@ -957,7 +1063,7 @@ int launch_quantize_unit(const QuantParams &p, hipStream_t stream) {
   int grid = 256 * (16 / waves_per_wg > 0 ? 16 / waves_per_wg : 1);
   if (tuning().quant_grid > 0) grid = tuning().quant_grid;
   if (grid > p.rows) grid = p.rows;
-  hipLaunchKernelGGL((quantize_rows_unit_kernel<FMT, MODE, SCALED>), dim3(grid), dim3(threads), lds, stream, p);
+  hipLaunchKernelGGL((quantize_rows_unit_kernel<FMT, MODE, SCALED, GROUPED>), dim3(grid), dim3(threads), lds, stream, p);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }
@@ -1212,6 +1318,51 @@ int swiglu_entry(const void *gate, const void *up, int ld, int rows, int K, cons
               : launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_SWIGLU, true>(p, st);
 }
 
+// grouped forms of reorder_quantize_x / swiglu_quantize_x: rows sorted by segment, segment offsets on the device
+int grouped_quantize_entry(int mode, const void *x, const void *up, int ld, int rows, int K, const int *seg, int n_seg,
+                           const int16_t *idx, int S, int fmt, const float *d_gscales, void *codes, void *scales,
+                           void *stream) {
+  if (fmt != ARCQ_FMT_NVFP4 && fmt != ARCQ_FMT_MXFP4) return ARCQ_ERR_FORMAT;
+  const int G = arcq_group_size(fmt);
+  if (rows < 0 || n_seg < 1 || K < 32 || K % 32 != 0 || K > 16384 || S < 0 || S > K || S % G != 0 || ld < K || ld % 8 != 0)
+    return ARCQ_ERR_SHAPE;
+  if (rows == 0) return ARCQ_OK;
+  if (!x || !seg || !idx || !codes || !scales || (mode == MODE_SWIGLU && !up)) return ARCQ_ERR_NULL;
+  if (!aligned16(x) || !aligned16(idx) || !aligned16(codes) || (mode == MODE_SWIGLU && !aligned16(up))) return ARCQ_ERR_ALIGN;
+  QuantParams p;
+  p.x = static_cast<const uint16_t *>(x);
+  p.up = static_cast<const uint16_t *>(up);
+  p.ldx = ld;
+  p.gamma = nullptr;
+  p.idx = idx;
+  p.codes = static_cast<uint8_t *>(codes);
+  p.scales = static_cast<uint8_t *>(scales);
+  p.d_gscale = d_gscales;
+  p.gscale = 1.0f;
+  p.eps = 0.0f;
+  p.rows = rows;
+  p.K = K;
+  p.S = S;
+  p.inv_k = 0.0;
+  p.seg = seg;
+  p.n_seg = n_seg;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool unit = d_gscales == nullptr;
+  if (mode == MODE_X) {
+    if (ld != K) return ARCQ_ERR_SHAPE;
+    if (fmt == ARCQ_FMT_NVFP4)
+      return unit ? launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_X, false, true>(p, st)
+                  : launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_X, true, true>(p, st);
+    return unit ? launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_X, false, true>(p, st)
+                : launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_X, true, true>(p, st);
+  }
+  if (fmt == ARCQ_FMT_NVFP4)
+    return unit ? launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_SWIGLU, false, true>(p, st)
+                : launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_SWIGLU, true, true>(p, st);
+  return unit ? launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_SWIGLU, false, true>(p, st)
+              : launch_quantize_unit<ARCQ_FMT_MXFP4, MODE_SWIGLU, true, true>(p, st);
+}
+
 }  // namespace
 }  // namespace arcq
 
@@ -1305,6 +1456,43 @@ int arcq_tensor_scale(const void *x, const void *up, int ld, int M, int K, float
   else
     hipLaunchKernelGGL(arcq::tensor_scale_kernel<false>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(x),
                        static_cast<const uint16_t *>(nullptr), (size_t)ld, M, K, divisor, ws, d_scale);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+int arcq_grouped_reorder_quantize_x(const void *x, int M, int K, const int *seg_offsets, int n_seg,
+                                    const int16_t *reorder_index, int select_num, int fmt, const float *d_global_scales,
+                                    void *codes, void *scales, void *stream) {
+  return arcq::grouped_quantize_entry(arcq::MODE_X, x, nullptr, K, M, K, seg_offsets, n_seg, reorder_index, select_num, fmt,
+                                      d_global_scales, codes, scales, stream);
+}
+
+int arcq_grouped_swiglu_quantize_x(const void *gate, const void *up, int ld, int M, int K, const int *seg_offsets, int n_seg,
+                                   const int16_t *reorder_index, int select_num, int fmt, const float *d_global_scales,
+                                   void *codes, void *scales, void *stream) {
+  return arcq::grouped_quantize_entry(arcq::MODE_SWIGLU, gate, up, ld, M, K, seg_offsets, n_seg, reorder_index, select_num,
+                                      fmt, d_global_scales, codes, scales, stream);
+}
+
+int arcq_grouped_tensor_scale(const void *x, const void *up, int ld, int M, int K, const int *seg_offsets, int n_seg,
+                              float divisor, float *d_scales, void *stream) {
+  if (M < 0 || n_seg < 1 || K < 8 || K % 8 != 0 || ld < K || ld % 8 != 0 || !(divisor > 0.0f)) return ARCQ_ERR_SHAPE;
+  if (!d_scales || !seg_offsets || (M > 0 && !x)) return ARCQ_ERR_NULL;
+  if (M > 0 && (!arcq::aligned16(x) || (up && !arcq::aligned16(up)))) return ARCQ_ERR_ALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint32_t *bits = reinterpret_cast<uint32_t *>(d_scales);
+  const int fin = (n_seg + 255) / 256;
+  hipLaunchKernelGGL(arcq::zero_words_kernel, dim3(fin), dim3(256), 0, st, bits, n_seg);
+  if (M > 0) {
+    const int grid = M < 2048 ? M : 2048;
+    if (up)
+      hipLaunchKernelGGL(arcq::grouped_absmax_kernel<true>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(x),
+                         static_cast<const uint16_t *>(up), (size_t)ld, M, K, seg_offsets, n_seg, bits);
+    else
+      hipLaunchKernelGGL(arcq::grouped_absmax_kernel<false>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(x),
+                         static_cast<const uint16_t *>(nullptr), (size_t)ld, M, K, seg_offsets, n_seg, bits);
+  }
+  hipLaunchKernelGGL(arcq::grouped_scale_finish_kernel, dim3(fin), dim3(256), 0, st, bits, n_seg, divisor);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }

@@ -21,8 +21,9 @@ What differs from the reference, on purpose:
     (model/qLlamaLayer.py:76).
   * quant_type 'MXFP4' runs the real kernels too; the reference falls back to fake-quantized bf16
     tensors and F.linear for it (model/qLinearLayer.py:71).
-  * the MoE block sorts tokens by expert on the device and reads the eight counts back once,
-    instead of one torch.where (a host sync) per expert.
+  * the MoE block sorts tokens by expert on the device and runs every step of the expert MLPs as one
+    grouped launch over all experts, with no read-back, instead of one torch.where (a host sync) and
+    five launches per expert.
 """
 from __future__ import annotations
 
@@ -494,14 +495,67 @@ class MixtralExpertMLP(nn.Module):
 
 class MixtralSparseMoeBlock(nn.Module):
     """model/qMixtralLayer.py:388-464: softmax router in fp32, top-k, renormalised weights, every
-    token processed by its experts without capacity limits."""
+    token processed by its experts without capacity limits.
 
-    def __init__(self, gate: nn.Linear, experts, top_k=2):
+    The reference walks the experts in Python (one torch.where, i.e. one host synchronisation, and five
+    launches per expert).  Here the (token, slot) pairs are sorted by expert on the device and each step of
+    the expert MLP is one grouped launch over all experts -- tensor scales, quantizer, w1|w3 GEMM, fused
+    SwiGLU quantizer, w2 GEMM -- reading the experts' row ranges from a device tensor: nothing is read back
+    to the host.  The experts' quantized weights are stacked for that; each expert module keeps views of
+    its part.  grouped=False keeps the per-expert loop (one read-back of the counts)."""
+
+    def __init__(self, gate: nn.Linear, experts, top_k=2, grouped=True):
         super().__init__()
         self.gate = gate
         self.experts = nn.ModuleList(experts)
         self.num_experts = len(experts)
         self.top_k = top_k
+        e0 = experts[0]
+        same = all(ex.w13.W.shape == e0.w13.W.shape and ex.w2.W.shape == e0.w2.W.shape and
+                   ex.quant_type == e0.quant_type and ex.w13.select_num == e0.w13.select_num and
+                   ex.w2.select_num == e0.w2.select_num and ex.w13.bias is None and ex.w2.bias is None
+                   for ex in experts)
+        kp13, kp2 = 2 * e0.w13.W.shape[1], 2 * e0.w2.W.shape[1]
+        self.grouped = bool(grouped) and same and kp13 % 128 == 0 and kp2 % 128 == 0 and min(kp13, kp2) >= 512 and \
+            e0.ffn <= 16384 and e0.ffn % 32 == 0 and e0.w13.in_features <= 16384
+        if self.grouped:
+            self.quant_type, self.ffn = e0.quant_type, e0.ffn
+            for name in ("w13", "w2"):
+                W = torch.stack([getattr(ex, name).W for ex in experts])
+                SF = torch.cat([getattr(ex, name).scale_w for ex in experts])
+                sc = torch.stack([getattr(ex, name).scale.reshape(()) for ex in experts]).to(torch.float32)
+                self.register_buffer(f"{name}_W", W)
+                self.register_buffer(f"{name}_scale_w", SF)
+                self.register_buffer(f"{name}_scale", sc)
+                per = SF.numel() // len(experts)
+                for i, ex in enumerate(experts):        # the experts keep views, not copies
+                    lin = getattr(ex, name)
+                    lin.W, lin.scale_w, lin.scale = W[i], SF[i * per:(i + 1) * per], sc[i]
+            self.register_buffer("w1_reorder_index", torch.stack([ex.w1_reorder_index for ex in experts]))
+            self.register_buffer("w2_reorder_index", torch.stack([ex.w2_reorder_index for ex in experts]))
+            self.register_buffer("_expert_ids", torch.arange(self.num_experts, device=W.device))
+
+    def _pair_ids(self, n, device):
+        if getattr(self, "_pairs", None) is None or self._pairs.numel() != n or self._pairs.device != device:
+            self._pairs = torch.arange(n, device=device)
+        return self._pairs
+
+    def _experts_grouped(self, xs, seg):
+        """the expert MLPs over tokens sorted by expert: xs bf16 [pairs, hidden], seg int32 [E+1] on the device"""
+        e0, qt = self.experts[0], self.quant_type
+        nv = qt == "NVFP4"
+        gs = agemm.grouped_tensor_scale(xs, seg, NVFP4_RANGE) if nv else None
+        q, sf = agemm.grouped_reorder_quantize_x(xs, seg, self.w1_reorder_index, e0.w13.select_num, fmt=qt,
+                                                 global_scales=gs)
+        h = agemm.grouped_matmul(q, self.w13_W, sf, self.w13_scale_w, seg, gs, self.w13_scale if nv else None, fmt=qt)
+        gate, up = h[:, :self.ffn], h[:, self.ffn:]
+        if nv:
+            q2, sf2, gs2 = agemm.grouped_swiglu_quantize_x(gate, up, seg, self.w2_reorder_index, e0.w2.select_num,
+                                                           fmt=qt, global_scales="absmax")
+        else:
+            q2, sf2 = agemm.grouped_swiglu_quantize_x(gate, up, seg, self.w2_reorder_index, e0.w2.select_num, fmt=qt)
+            gs2 = None
+        return agemm.grouped_matmul(q2, self.w2_W, sf2, self.w2_scale_w, seg, gs2, self.w2_scale if nv else None, fmt=qt)
 
     @torch.no_grad()
     def forward(self, hidden_states, router_logits: Optional[torch.Tensor] = None):
@@ -516,10 +570,23 @@ class MixtralSparseMoeBlock(nn.Module):
         flat_e = sel.reshape(-1)
         order = torch.argsort(flat_e, stable=True)
         tok = order // self.top_k
-        counts = torch.bincount(flat_e, minlength=self.num_experts).tolist()   # the one host read-back
         xs = x.index_select(0, tok)
         ws = w.reshape(-1).index_select(0, order)
+        if self.grouped:
+            counts = (flat_e[:, None] == self._expert_ids[None, :]).sum(0)      # on the device: no read-back
+            seg = torch.zeros(self.num_experts + 1, dtype=torch.int32, device=x.device)
+            seg[1:] = torch.cumsum(counts, 0)
+            y = self._experts_grouped(xs, seg)
+            if hid % 8 == 0 and self.top_k <= 8:
+                position = torch.empty_like(order)
+                position[order] = self._pair_ids(order.numel(), x.device)        # inverse of the sort
+                return agemm.moe_combine(y, position, ws.contiguous(), x.shape[0], self.top_k).reshape(bsz, q_len, hid), \
+                    router_logits
+            out = torch.zeros_like(x)
+            out.index_add_(0, tok, (y * ws[:, None]).to(x.dtype))
+            return out.reshape(bsz, q_len, hid), router_logits
         out = torch.zeros_like(x)
+        counts = torch.bincount(flat_e, minlength=self.num_experts).tolist()   # the one host read-back
         beg = 0
         for e, n in enumerate(counts):
             if n == 0:
@@ -531,7 +598,7 @@ class MixtralSparseMoeBlock(nn.Module):
 
 
 def build_mixtral_block(hidden=4096, ffn=14336, num_experts=8, top_k=2, select_num=128, quant_type="NVFP4",
-                        indices=None, seed=5, device="cuda"):
+                        indices=None, seed=5, device="cuda", grouped=True):
     """Random-weight MoE block of benchmark configuration 5; `indices[e]` = (input index, w2 index)."""
     gen = torch.Generator().manual_seed(seed)
     gate = _linear(num_experts, hidden, 1.0 / math.sqrt(hidden), device, gen)
@@ -547,7 +614,7 @@ def build_mixtral_block(hidden=4096, ffn=14336, num_experts=8, top_k=2, select_n
             i_w2 = torch.arange(ffn, dtype=torch.int16, device=device)
         experts.append(MixtralExpertMLP(w1, w3, w2, select_num, i_in, i_w2, quant_type))
         del w1, w3, w2
-    return MixtralSparseMoeBlock(gate, experts, top_k)
+    return MixtralSparseMoeBlock(gate, experts, top_k, grouped=grouped)
 
 
 class GraphedDecodeStep:

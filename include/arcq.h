@@ -198,6 +198,60 @@ size_t arcq_matmul_noalloc_limit(void);
 size_t arcq_matmul_scratch_bytes(int M, int N, int Kp, int fmt);
 
 /*
+ * Grouped launches for mixture-of-experts blocks.  The reference walks the experts in Python
+ * (model/qMixtralLayer.py:458-471): per expert one torch.where (a host synchronisation), a gather of its
+ * tokens, reorder_quantize_x with the expert's reorder_index (:530), two GEMMs against the expert's
+ * weights, the activation quantizer again (:539) and the last GEMM.  Here the tokens are sorted by expert
+ * once and each of those steps is ONE launch over all experts:
+ *   seg_offsets  int32 [n_seg+1] on the device: rows seg_offsets[e] .. seg_offsets[e+1]-1 of the sorted
+ *                activations belong to expert e (non-decreasing, seg_offsets[0] = 0, seg_offsets[n_seg] <= M;
+ *                an expert may own no row; rows behind the last segment are left untouched)
+ *   reorder_index      int16 [n_seg, K]: one channel order per expert
+ *   d_global_scales    fp32 [n_seg] on the device: one NVFP4 tensor scale per expert (max |x_e| / 2688,
+ *                      model/qLlamaLayer.py:73-77 applied to the expert's tokens as model/qMixtralLayer.py:530
+ *                      does), or NULL for tensor scale 1 everywhere (MXFP4)
+ * Nothing is read back to the host.  Codes and scale bytes of a row are those arcq_reorder_quantize_x /
+ * arcq_swiglu_quantize_x write for that row with its expert's index and scale.
+ * arcq_grouped_tensor_scale writes the n_seg scales (1 for an expert without rows or with only zeros);
+ * `up` as for arcq_tensor_scale.  K <= 16384 for the quantizers.
+ */
+int arcq_grouped_reorder_quantize_x(const void *x, int M, int K, const int *seg_offsets, int n_seg,
+                                    const int16_t *reorder_index, int select_num, int fmt, const float *d_global_scales,
+                                    void *codes, void *scales, void *stream);
+int arcq_grouped_swiglu_quantize_x(const void *gate, const void *up, int ld, int M, int K, const int *seg_offsets, int n_seg,
+                                   const int16_t *reorder_index, int select_num, int fmt, const float *d_global_scales,
+                                   void *codes, void *scales, void *stream);
+int arcq_grouped_tensor_scale(const void *x, const void *up, int ld, int M, int K, const int *seg_offsets, int n_seg,
+                              float divisor, float *d_scales, void *stream);
+/*
+ * Grouped GEMM: rows seg_offsets[e] .. seg_offsets[e+1]-1 of C = alpha * alpha_a[e] * alpha_b[e] *
+ * dq(A rows of e) @ dq(B_e)^T with expert e's weights B_e = b_codes + e * N * Kp/2 (scales likewise:
+ * the experts' quantized weights stacked [n_seg, N, ...]).  One launch; every workgroup finds its
+ * expert and tile from seg_offsets on the device.  Replaces the per-expert agemm.matmul calls of
+ * model/qMixtralLayer.py:466-543 -> model/qLinearLayer.py:65-81.
+ *   d_alpha_a, d_alpha_b  fp32 [n_seg] on the device or NULL (activation / weight tensor scales per expert)
+ *   residual              NULL or bf16 [M, N], added as by arcq_matmul_add
+ *   Kp                    multiple of 128, >= 512; scale arrays 16-byte aligned (else ARCQ_ERR_SHAPE / _ALIGN)
+ */
+int arcq_grouped_matmul(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                        const int *seg_offsets, int n_seg, int M, int N, int Kp, int fmt, float alpha,
+                        const float *d_alpha_a, const float *d_alpha_b, const void *residual, void *c, void *stream);
+
+/*
+ * Last step of a mixture-of-experts block: out[t] = sum over token t's experts, in ascending expert number, of
+ * bf16(y[row] * weight[row]), every partial sum rounded to bf16 -- what model/qMixtralLayer.py:466-471 gets
+ * from `expert(x) * routing_weights[...]` followed by final_hidden_states.index_add_ per expert.  One launch,
+ * one read of every expert-output row, no atomics (reproducible).
+ *   y         bf16 [pairs, H]: the expert outputs in expert-sorted row order (arcq_grouped_matmul's output)
+ *   position  int64 [tokens * top_k] on the device: row of y holding token t's j-th expert (the inverse of the
+ *             sort order); entries outside [0, pairs) contribute nothing
+ *   weight    bf16 [pairs]: router weights in the same sorted order
+ *   H multiple of 8, top_k <= 8
+ */
+int arcq_moe_combine(const void *y, const int64_t *position, const void *weight, int tokens, int H, int top_k, int pairs,
+                     void *out, void *stream);
+
+/*
  * INT4 paged KV cache (the reference's decode-attention path: agemm.init_kv_i4 / append_kv_i4 /
  * batch_decode_i4, kernels/src/bindings.cpp:287-413 -> kernels/src/flashinfer.cu:9-112, with the
  * torch-side quantizer asym_quantize_and_pack_i4, model/kv_cache.py:23-37, fused into the append).

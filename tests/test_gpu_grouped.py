@@ -1,0 +1,190 @@
+"""Grouped operators for mixture-of-experts blocks (tokens sorted by expert, one launch per step for all
+experts, segment offsets on the device) against the per-expert path they replace:
+
+* grouped quantizer: codes and scale bytes of every row bit-exact against the C oracle's quantizer run
+  on that expert's rows with that expert's reorder_index and tensor scale (model/qMixtralLayer.py:530);
+* grouped fused SwiGLU quantizer: bit-identical to the ungrouped operator on each expert's rows;
+* grouped GEMM: against the fp64 oracle with each expert's weights (model/qMixtralLayer.py:466-543).
+"""
+import numpy as np
+import pytest
+import torch
+
+import recipes
+
+pytestmark = pytest.mark.gpu
+FMTS = ["NVFP4", "MXFP4"]
+
+
+@pytest.fixture(scope="module")
+def agemm():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from arcquant_amd import agemm as m
+    return m
+
+
+def rel_fro(got, want):
+    got, want = got.double(), want.double()
+    return float((got - want).norm() / want.norm())
+
+
+def segments(counts):
+    return torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32)
+
+
+def expert_scale(t):
+    """max|t| / 2688 as the callers compute it in fp32 (model/qLlamaLayer.py:74); 1 for no rows / all zeros"""
+    if t.numel() == 0:
+        return 1.0
+    s = float(t.abs().max().float() / torch.tensor(2688.0))
+    return s if s != 0.0 else 1.0
+
+
+COUNTS = [[5, 0, 17, 1, 300, 0, 64, 9], [40], [0, 0, 3], [130, 131, 2, 700]]
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("counts", COUNTS)
+@pytest.mark.parametrize("K,S", [(4096, 128), (512, 512), (1024, 0)])
+def test_grouped_quantize_matches_per_expert_oracle(agemm, oracle, fmt, counts, K, S):
+    T, E = sum(counts), len(counts)
+    x = recipes.activations(T, K, seed=7000 + T + K, outlier_frac=0.01, outlier_gain=40.0)
+    seg = segments(counts)
+    # per-expert channel order from the per-expert channel maxima (experts without rows: a random order)
+    g = torch.Generator().manual_seed(E + K)
+    idx = torch.stack([recipes.reorder_index(x[seg[e]:seg[e + 1]]) if counts[e] else
+                       torch.randperm(K, generator=g).to(torch.int16) for e in range(E)])
+    for e in range(E):                      # per-expert magnitudes, so that the tensor scales differ
+        x[seg[e]:seg[e + 1]] *= (1.0 + 0.5 * e)
+    x = x.to(torch.bfloat16)
+    print(f"grouped quantize {fmt} counts={counts} K={K} S={S}", flush=True)
+    gs = None
+    if fmt == "NVFP4":
+        gs = agemm.grouped_tensor_scale(x.cuda(), seg.cuda())
+        want_gs = [expert_scale(x[seg[e]:seg[e + 1]]) for e in range(E)]
+        assert gs.cpu().tolist() == pytest.approx(want_gs, rel=0, abs=0)
+    q, sf = agemm.grouped_reorder_quantize_x(x.cuda(), seg.cuda(), idx.cuda(), S, fmt=fmt, global_scales=gs)
+    q, sf = q.cpu().numpy(), sf.cpu().numpy().reshape(T, -1)
+    for e in range(E):
+        if not counts[e]:
+            continue
+        lo, hi = int(seg[e]), int(seg[e + 1])
+        want = oracle.quantize_x(x[lo:hi], idx[e], S, fmt, 1.0 if gs is None else float(gs[e]))
+        assert np.array_equal(sf[lo:hi], want["scales"]), f"expert {e}: scale bytes differ"
+        assert np.array_equal(q[lo:hi], want["codes"]), f"expert {e}: codes differ"
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("counts", [[5, 0, 17, 1, 300, 0, 64, 9], [700, 3]])
+def test_grouped_swiglu_matches_ungrouped(agemm, fmt, counts):
+    T, E, F, S = sum(counts), len(counts), 1024, 128
+    g = torch.Generator().manual_seed(T)
+    gu = (torch.randn(T, 2 * F, generator=g) * 2.0).to(torch.bfloat16).cuda()
+    seg = segments(counts)
+    for e in range(E):
+        gu[seg[e]:seg[e + 1]] *= (1.0 + 0.25 * e)
+    idx = torch.stack([torch.randperm(F, generator=g).to(torch.int16) for _ in range(E)]).cuda()
+    gate, up = gu[:, :F], gu[:, F:]
+    print(f"grouped swiglu {fmt} counts={counts}", flush=True)
+    if fmt == "NVFP4":
+        q, sf, gs = agemm.grouped_swiglu_quantize_x(gate, up, seg.cuda(), idx, S, fmt=fmt, global_scales="absmax")
+    else:
+        q, sf = agemm.grouped_swiglu_quantize_x(gate, up, seg.cuda(), idx, S, fmt=fmt)
+    sf = sf.view(T, -1)
+    for e in range(E):
+        lo, hi = int(seg[e]), int(seg[e + 1])
+        if lo == hi:
+            if fmt == "NVFP4":
+                assert float(gs[e]) == 1.0
+            continue
+        if fmt == "NVFP4":
+            wq, wsf, wgs = agemm.swiglu_quantize_x(gate[lo:hi], up[lo:hi], idx[e], S, fmt=fmt, global_scale="absmax")
+            assert float(wgs) == float(gs[e])
+        else:
+            wq, wsf = agemm.swiglu_quantize_x(gate[lo:hi], up[lo:hi], idx[e], S, fmt=fmt)
+        assert torch.equal(sf[lo:hi], wsf.view(hi - lo, -1)) and torch.equal(q[lo:hi], wq), f"expert {e}"
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("counts,N,K,S", [([5, 0, 17, 1, 300, 0, 64, 9], 384, 512, 128),
+                                           ([40], 256, 1024, 0),
+                                           ([0, 0, 3], 130, 448, 64),
+                                           ([130, 131, 2, 700], 512, 896, 128),
+                                           ([300, 500, 10], 512, 512, 128),
+                                           ([1100, 900], 256, 512, 0),
+                                           ([2500, 2100], 256, 512, 0)])
+def test_grouped_matmul_matches_oracle(agemm, oracle, fmt, counts, N, K, S):
+    """The launch picks its tile from the average rows per expert: these cases take the 128x64, 128x128
+    and 256x256 tiles; experts without rows, with one row, with ragged last tiles; the residual form as well."""
+    T, E = sum(counts), len(counts)
+    x = recipes.activations(T, K, seed=8000 + T + N, outlier_frac=0.01, outlier_gain=40.0)
+    seg = segments(counts)
+    g = torch.Generator().manual_seed(N + K)
+    idx = torch.stack([torch.randperm(K, generator=g).to(torch.int16) for _ in range(E)])
+    w = [recipes.weights(N, K, seed=8100 + e, std=0.02 * (1 + e)) for e in range(E)]
+    print(f"grouped matmul {fmt} counts={counts} N={N} K={K} S={S}", flush=True)
+    gs = agemm.grouped_tensor_scale(x.cuda(), seg.cuda()) if fmt == "NVFP4" else None
+    a, sfa = agemm.grouped_reorder_quantize_x(x.cuda(), seg.cuda(), idx.cuda(), S, fmt=fmt, global_scales=gs)
+    bq, bsf, gw = [], [], []
+    for e in range(E):
+        s = recipes.tensor_scale(w[e], fmt)
+        b, sfb = agemm.reorder_quantize_w(w[e].cuda(), idx[e].cuda(), S, fmt=fmt, global_scale=s)
+        bq.append(b), bsf.append(sfb), gw.append(s)
+    B, SFB = torch.stack(bq), torch.cat(bsf)
+    gw_d = torch.tensor(gw, dtype=torch.float32).cuda() if fmt == "NVFP4" else None
+    res = (torch.randn(T, N, generator=g)).to(torch.bfloat16).cuda()
+    y = agemm.grouped_matmul(a, B, sfa, SFB, seg.cuda(), gs, gw_d)
+    y2 = agemm.grouped_matmul(a, B, sfa, SFB, seg.cuda(), gs, gw_d, residual=res)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, (y + res))
+    ac, asc = a.cpu().numpy(), sfa.cpu().numpy().reshape(T, -1)
+    for e in range(E):
+        lo, hi = int(seg[e]), int(seg[e + 1])
+        if lo == hi:
+            continue
+        alpha = (float(gs[e]) * gw[e]) if fmt == "NVFP4" else 1.0
+        want = oracle.matmul(ac[lo:hi], asc[lo:hi], bq[e].cpu().numpy(), bsf[e].cpu().numpy().reshape(N, -1), fmt, alpha=alpha)
+        assert rel_fro(y[lo:hi].float().cpu(), torch.from_numpy(want)) < 1e-2, f"expert {e}"
+        assert torch.allclose(y[lo:hi].float().cpu(), torch.from_numpy(want).float(), rtol=2 ** -7,
+                              atol=1e-3 * float(np.abs(want).max())), f"expert {e}"
+
+
+def test_grouped_matmul_ignores_rows_behind_the_last_segment(agemm):
+    """seg[E] < M: the rows behind it are not written; offsets that shrink or leave the tensor read as empty segments"""
+    T, N, K, S, fmt = 200, 256, 512, 0, "MXFP4"
+    x = recipes.activations(T, K, seed=1).cuda()
+    idx = torch.arange(K, dtype=torch.int16).cuda()
+    a, sfa = agemm.reorder_quantize_x(x, idx, S, fmt=fmt)
+    b, sfb = agemm.reorder_quantize_w(recipes.weights(N, K, seed=2).cuda(), idx, S, fmt=fmt)
+    whole = agemm.matmul(a, b, sfa, sfb, 1.0, fmt=fmt)
+    B, SFB = torch.stack([b, b]), torch.cat([sfb, sfb])
+    for seg in ([0, 100, 150], [0, 300, 100], [0, -5, 200]):
+        y = agemm.grouped_matmul(a, B, sfa, SFB, torch.tensor(seg, dtype=torch.int32).cuda())
+        end = max(0, min(seg[1], T))
+        end = max(end, min(seg[2], T))
+        assert torch.equal(y[:end], whole[:end]), seg
+
+
+@pytest.mark.parametrize("top_k", [1, 2, 3])
+def test_moe_combine_matches_index_add(agemm, top_k):
+    """weights applied and expert outputs summed per token as model/qMixtralLayer.py:466-471 does: expert after
+    expert in ascending number into a bf16 tensor of zeros"""
+    tokens, H, E = 300, 1032, 6
+    g = torch.Generator().manual_seed(top_k)
+    sel = torch.stack([torch.randperm(E, generator=g)[:top_k] for _ in range(tokens)])
+    w = torch.rand(tokens, top_k, generator=g).to(torch.bfloat16)
+    flat = sel.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    tok = order // top_k
+    y = torch.randn(tokens * top_k, H, generator=g).to(torch.bfloat16)
+    ws = w.reshape(-1)[order]
+    want = torch.zeros(tokens, H, dtype=torch.bfloat16)
+    counts = torch.bincount(flat, minlength=E).tolist()
+    beg = 0
+    for e, n in enumerate(counts):                 # the reference's loop over experts
+        want.index_add_(0, tok[beg:beg + n], y[beg:beg + n] * ws[beg:beg + n, None])
+        beg += n
+    position = torch.empty_like(order)
+    position[order] = torch.arange(order.numel())
+    got = agemm.moe_combine(y.cuda(), position.cuda(), ws.cuda(), tokens, top_k)
+    assert torch.equal(got.cpu(), want)

@@ -134,14 +134,21 @@ def test_decoder_layer_matches_fake_quant_flow(layers, fq, fmt):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-def test_mixtral_block_matches_reference_loop(layers, fq, fmt):
-    hidden, ffn, E, S = 256, 512, 4, 64
+@pytest.mark.parametrize("grouped", [True, False])
+def test_mixtral_block_matches_reference_loop(layers, fq, fmt, grouped):
+    """The MoE block, as grouped launches over all experts and as the per-expert loop, against the
+    reference's loop (model/qMixtralLayer.py:441-471) on the CPU; every expert has its own channel orders."""
+    hidden, ffn, E, S = 384, 512, 4, 128
     tokens = 96
-    block = layers.build_mixtral_block(hidden, ffn, E, 2, S, fmt, seed=5)
     g = torch.Generator().manual_seed(9)
+    indices = [(torch.randperm(hidden, generator=g).to(torch.int16).cuda(),
+                torch.randperm(ffn, generator=g).to(torch.int16).cuda()) for _ in range(E)]
+    block = layers.build_mixtral_block(hidden, ffn, E, 2, S, fmt, indices=indices, seed=5, grouped=grouped)
+    assert block.grouped == grouped
     x = torch.randn(1, tokens, hidden, generator=g).to(torch.bfloat16)
     logits = torch.randn(tokens, E, generator=g)
     logits[:, 3] -= 100.0                                   # an expert that receives no token
+    print(f"mixtral block {fmt} grouped={grouped}", flush=True)
     y, _ = block(x.cuda(), router_logits=logits.cuda())
     assert y.shape == x.shape
 
@@ -152,14 +159,14 @@ def test_mixtral_block_matches_reference_loop(layers, fq, fmt):
     w = (w / w.sum(dim=-1, keepdim=True)).to(torch.bfloat16)
     want = torch.zeros(tokens, hidden, dtype=torch.bfloat16)
     x2 = x.view(tokens, hidden)
-    ih, ii = torch.arange(hidden), torch.arange(ffn)
     for e in range(E):
         slot, top_x = torch.where((sel == e).T)
         if top_x.numel() == 0:
             continue
         ex = block.experts[e]
-        w13 = (agemm.dequantize(ex.w13.W, ex.w13.scale_w, fmt=fmt) * ex.w13.scale).cpu()
-        w2 = (agemm.dequantize(ex.w2.W, ex.w2.scale_w, fmt=fmt) * ex.w2.scale).cpu()
+        ih, ii = indices[e][0].cpu(), indices[e][1].cpu()
+        w13 = (agemm.dequantize(ex.w13.W.contiguous(), ex.w13.scale_w.contiguous(), fmt=fmt) * ex.w13.scale).cpu()
+        w2 = (agemm.dequantize(ex.w2.W.contiguous(), ex.w2.scale_w.contiguous(), fmt=fmt) * ex.w2.scale).cpu()
         cur = x2[top_x]
         hcur = (ref_quant_x(fq, cur, ih, S, fmt) @ w13.T).to(torch.bfloat16)
         t = F.silu(hcur[:, :ffn]) * hcur[:, ffn:]
@@ -167,6 +174,38 @@ def test_mixtral_block_matches_reference_loop(layers, fq, fmt):
         want.index_add_(0, top_x, out * w[top_x, slot, None])
     assert rel_fro(y.view(tokens, hidden), want) < 2e-2
     assert float(y.abs().sum()) > 0
+
+
+def test_mixtral_block_grouped_equals_loop_at_benchmark_size(layers):
+    """Benchmark configuration 5: 8 experts, top-2, hidden 4096, intermediate 14336, 4096 tokens routed with
+    a Zipf(1.1) skew over the experts, per-expert channel orders from the per-expert channel maxima,
+    select_num 128, NVFP4.  The grouped launches against the per-expert loop of the same block (same
+    quantized weights): the quantizers are bit-identical, the GEMMs differ in tile shape only."""
+    hidden, ffn, E, S, tokens, fmt = 4096, 14336, 8, 128, 4096, "NVFP4"
+    g = torch.Generator().manual_seed(55)
+    x = recipes.activations(tokens, hidden, seed=5, outlier_frac=0.01, outlier_gain=40.0)
+    zipf = 1.0 / torch.arange(1, E + 1, dtype=torch.float32) ** 1.1
+    logits = torch.log(zipf)[None, :] + torch.randn(tokens, E, generator=g)
+    sel = torch.topk(torch.softmax(logits, 1), 2, dim=-1).indices
+    indices = []
+    for e in range(E):
+        mine = x[(sel == e).any(1)]
+        i_in = recipes.reorder_index(mine if mine.numel() else x).cuda()
+        indices.append((i_in, torch.randperm(ffn, generator=g).to(torch.int16).cuda()))
+    block = layers.build_mixtral_block(hidden, ffn, E, 2, S, fmt, indices=indices, seed=5, grouped=True)
+    assert block.grouped
+    xc, lc = x.cuda().view(1, tokens, hidden), logits.cuda()
+    print("mixtral block at configuration 5 size: grouped", flush=True)
+    y_grouped, _ = block(xc, router_logits=lc)
+    torch.cuda.synchronize()
+    block.grouped = False
+    print("mixtral block at configuration 5 size: per-expert loop", flush=True)
+    y_loop, _ = block(xc, router_logits=lc)
+    torch.cuda.synchronize()
+    counts = torch.bincount(sel.reshape(-1), minlength=E).tolist()
+    assert max(counts) > 3 * min(counts)                     # the skew is there
+    assert rel_fro(y_grouped, y_loop) < 5e-3                 # bf16 roundings of differently ordered fp32 sums
+    assert float(y_loop.abs().sum()) > 0
 
 
 @pytest.mark.parametrize("fmt", FMTS)
