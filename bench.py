@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ARC quantized-linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--gemm-table] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--headline-only] [--no-cpu]
 
 Prints ONE JSON line.  A "step" is one launch of the fused RMSNorm + reorder + quantize kernel
 over one batch of synthetic activations already resident in HBM: M=4096 tokens, hidden 4096,
@@ -13,8 +13,15 @@ Cache, so the rate is an HBM rate, not a cache rate.
   roofline       the same kernel against the 8 TB/s HBM peak, from HIP events around each launch
   cpu_baseline   the reference's fake-quant arithmetic (torch restatement, oracle/fakequant_torch.py)
                  timed on this box's host cores on a bounded sample of the same workload
-  gemm           ARC FP4 GEMM TFLOP/s at Llama-3-8B shapes next to torch's bf16 GEMM of the same
-                 (M, N, K'), outside the timed region (--gemm-table for every shape x M)
+  quantize       benchmark configuration 2 in full: fused norm at M in {1, 16, 256, 4096}, select_num in
+                 {64, 256}, both formats, plus the plain quantizers at M = 4096
+  gemm           benchmark configuration 3 in full: ARC FP4 GEMM at the four Llama-3-8B projection shapes
+                 x M in {1, 16, 128, 512, 2048, 4096}, both formats, next to torch's bf16 GEMM of the same
+                 (M, N, K'), each with its fraction of the MFMA peak
+  layers         benchmark configurations 4 and 5: a decoder layer (prefill 8 x 2048, decode batch 64) and a
+                 Mixtral MoE block, reorder indices from channel maxima, next to the same layer in bf16
+Everything but the headline step sits outside the timed region.  --quick drops the layer rows and half of
+the GEMM rows; --headline-only (for counter runs) keeps the headline kernel and the copy kernels only.
 """
 from __future__ import annotations
 
@@ -33,10 +40,25 @@ MFMA_PEAK_TFLOPS = {"MXFP4": 10100.0, "NVFP4": 2500.0, "bf16": 2500.0}   # dense
 
 H, M_TOKENS, SELECT, EPS = 4096, 4096, 256, 1e-5
 FMT = "NVFP4"
-# HBM bytes per launch of the headline kernel on this workload from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (two runs), each scaled by what the same counter reads for arcq_stream_probe moving a known
-# number of bytes (profiles/bench_quantize_and_gemm_kernels.md): 33.74 MB fetched + 10.09 MB written.
-MEASURED_TRAFFIC_BYTES = 43_830_000
+# HBM bytes per launch of the headline kernel come from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two
+# runs), each scaled by what the same counter reads for arcq_stream_probe moving a known number of bytes.
+# The summary of those runs under profiles/ carries the figure on a line of its own together with the
+# kernel and the workload it was measured on; it is taken from there, and only for that workload.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "rmsnorm_quantize_nvfp4_4096x4096_hbm_traffic.md")
+
+
+def measured_traffic(workload_key):
+    """(bytes per launch, kernel, source file) from the committed counter summary, or (None, None, None)
+    when it is absent or covers another workload"""
+    import re
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, None, None
+    m = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)\s*;\s*kernel\s*=\s*(.+?)\s*;\s*workload\s*=\s*(.+?)\s*$", text, re.M)
+    if not m or m.group(3) != workload_key:
+        return None, None, None
+    return int(m.group(1)), m.group(2), os.path.relpath(TRAFFIC_PROFILE, ROOT)
 
 
 def quant_bytes(M, K, S, fmt, fused_norm):
@@ -145,7 +167,8 @@ def gemm_rows(torch, agemm, shapes, Ms, fmts, iters=40):
             for i in range(5):
                 fn(i)
             ms = loop_time_ms(fn, iters, torch)
-            row["bf16_torch"] = {"us": round(ms * 1e3, 2), "tflops": round(gemm_flops(M, N, Kp) / ms / 1e9, 1)}
+            row["bf16_torch"] = {"us": round(ms * 1e3, 2), "tflops": round(gemm_flops(M, N, Kp) / ms / 1e9, 1),
+                                 "frac_of_mfma_peak": round(gemm_flops(M, N, Kp) / ms / 1e9 / MFMA_PEAK_TFLOPS["bf16"], 4)}
             for f in fmts:
                 row[f]["vs_bf16"] = round(row["bf16_torch"]["us"] / row[f]["us"], 2)
             rows.append(row)
@@ -160,8 +183,10 @@ def layer_rows(torch, iters=10):
     (torch: hipBLASLt GEMMs, the same SDPA).  One decoder layer of Llama-3-8B geometry (hidden 4096,
     32 query / 8 KV heads of 128, SwiGLU 14336, fused qkv and gate_up), prefill 8 x 2048 tokens and a
     decode step of batch 64 over a 2048-token KV cache; one Mixtral MoE block (8 experts, top-2,
-    4096 tokens, expert popularity Zipf(1.1))."""
+    4096 tokens, expert popularity Zipf(1.1)).  Reorder indices are the ascending order of the per-channel
+    maxima of each linear's input, taken from one bf16 pass over the same activations."""
     import torch.nn.functional as F
+    import recipes
     from arcquant_amd import layers
     rows = []
     hidden, inter, nh, nkv, eps = 4096, 14336, 32, 8, 1e-5
@@ -184,31 +209,49 @@ def layer_rows(torch, iters=10):
         h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + eps)
         return w * h.to(x.dtype)
 
+    def channel_order(t):
+        return torch.argsort(t.reshape(-1, t.shape[-1]).float().abs().amax(0), stable=True).to(torch.int16)
+
+    def bf16_layer(W, g1, g2, x, kv=None, past=0, taps=None):
+        b, s, _ = x.shape
+        n1 = rms(x, g1)
+        qkv = F.linear(n1, W["qkv"])
+        q = qkv[..., :nh * d].view(b, s, nh, d).transpose(1, 2)
+        k = qkv[..., nh * d:(nh + nkv) * d].view(b, s, nkv, d).transpose(1, 2)
+        v = qkv[..., (nh + nkv) * d:].view(b, s, nkv, d).transpose(1, 2)
+        q, k = layers.rotary_pos_emb(q, k, past)
+        if kv is not None:
+            kv[0][:, :, past:past + s] = k
+            kv[1][:, :, past:past + s] = v
+            k, v = kv[0][:, :, :past + s], kv[1][:, :, :past + s]
+        o = F.scaled_dot_product_attention(q, k, v, is_causal=(s > 1 and past == 0), enable_gqa=True)
+        o = o.transpose(1, 2).reshape(b, s, hidden)
+        h = x + F.linear(o, W["o"])
+        n2 = rms(h, g2)
+        gu = F.linear(n2, W["gate_up"])
+        t = F.silu(gu[..., :inter]) * gu[..., inter:]
+        if taps is not None:
+            taps.update(attn_in=channel_order(n1), o_in=channel_order(o), mlp_in=channel_order(n2), down_in=channel_order(t))
+        return h + F.linear(t, W["down"])
+
     for fmt in ("MXFP4", "NVFP4"):
-        layer = layers.LlamaDecoderLayer(hidden, inter, nh, nkv, eps=eps, select_num=256, select_num_down=256,
+        # the layer is built twice: once with identity orders to get at its weights, which one bf16 pass turns
+        # into the channel orders (the calibration the reference runs offline), then with those orders
+        x = hidden_states(8, 2048)
+        probe = layers.LlamaDecoderLayer(hidden, inter, nh, nkv, eps=eps, select_num=256, select_num_down=256,
                                          quant_type=fmt, seed=4)
+        W = {k: v.weight.data for k, v in probe.linears.items()}
+        g1, g2 = probe.input_layernorm.weight, probe.post_attention_layernorm.weight
+        taps = {}
+        bf16_layer(W, g1, g2, x[:2], taps=taps)
+        del probe
+        layer = layers.LlamaDecoderLayer(hidden, inter, nh, nkv, eps=eps, select_num=256, select_num_down=256,
+                                         quant_type=fmt, seed=4, indices={k: v.cuda() for k, v in taps.items()})
         W = {k: v.weight.data for k, v in layer.linears.items()}
         g1, g2 = layer.input_layernorm.weight, layer.post_attention_layernorm.weight
 
-        def bf16_layer(x, kv=None, past=0):
-            b, s, _ = x.shape
-            qkv = F.linear(rms(x, g1), W["qkv"])
-            q = qkv[..., :nh * d].view(b, s, nh, d).transpose(1, 2)
-            k = qkv[..., nh * d:(nh + nkv) * d].view(b, s, nkv, d).transpose(1, 2)
-            v = qkv[..., (nh + nkv) * d:].view(b, s, nkv, d).transpose(1, 2)
-            q, k = layers.rotary_pos_emb(q, k, past)
-            if kv is not None:
-                kv[0][:, :, past:past + s] = k
-                kv[1][:, :, past:past + s] = v
-                k, v = kv[0][:, :, :past + s], kv[1][:, :, :past + s]
-            o = F.scaled_dot_product_attention(q, k, v, is_causal=(s > 1 and past == 0), enable_gqa=True)
-            h = x + F.linear(o.transpose(1, 2).reshape(b, s, hidden), W["o"])
-            gu = F.linear(rms(h, g2), W["gate_up"])
-            return h + F.linear(F.silu(gu[..., :inter]) * gu[..., inter:], W["down"])
-
-        x = hidden_states(8, 2048)
         ms_arc = timed(lambda: layer(x))
-        ms_bf = timed(lambda: bf16_layer(x))
+        ms_bf = timed(lambda: bf16_layer(W, g1, g2, x))
         rows.append({"config": "decoder layer prefill 8x2048", "fmt": fmt, "arc_ms": round(ms_arc, 3),
                      "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_arc, 2),
                      "tokens_per_s": round(8 * 2048 / ms_arc * 1e3)})
@@ -219,8 +262,19 @@ def layer_rows(torch, iters=10):
               torch.randn(64, nkv, kvlen + 8, d, device="cuda", dtype=torch.bfloat16))
         x = hidden_states(64, 1)
         ms_arc = timed(lambda: layer(x, kv, kvlen))
-        ms_bf = timed(lambda: bf16_layer(x, kv, kvlen))
-        rows.append({"config": f"decoder layer decode batch 64, KV length {kvlen}", "fmt": fmt,
+        ms_bf = timed(lambda: bf16_layer(W, g1, g2, x, kv, kvlen))
+        # the bf16 step as a HIP graph too, so that a graphed ARC step below is compared like with like
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                bf16_layer(W, g1, g2, x, kv, kvlen)
+        torch.cuda.current_stream().wait_stream(side)
+        bf_graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(bf_graph, stream=side):
+            bf16_layer(W, g1, g2, x, kv, kvlen)
+        ms_bf_graph = timed(bf_graph.replay)
+        rows.append({"config": f"decoder layer decode batch 64, KV length {kvlen}, bf16 KV cache + SDPA, eager", "fmt": fmt,
                      "arc_ms": round(ms_arc, 3), "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_arc, 2),
                      "tokens_per_s": round(64 / ms_arc * 1e3)})
         print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
@@ -234,34 +288,46 @@ def layer_rows(torch, iters=10):
             cache._specs["last_page_offset"].fill_(kvlen % 16 or 16)
             return layer(x, cache, kvlen)
         ms_i4 = timed(paged_step)
-        rows.append({"config": f"decoder layer decode batch 64, KV length {kvlen}, INT4 paged KV cache", "fmt": fmt,
+        rows.append({"config": f"decoder layer decode batch 64, KV length {kvlen}, INT4 paged KV cache, eager", "fmt": fmt,
                      "arc_ms": round(ms_i4, 3), "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_i4, 2),
                      "tokens_per_s": round(64 / ms_i4 * 1e3)})
         print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
         # ... and the whole step replayed from a captured HIP graph (the KV length grows by one per
-        # replay, as in generation: 2048 -> ~2060 over the timed repetitions)
+        # replay, as in generation: 2048 -> ~2060 over the timed repetitions), against the graphed bf16 step
         cache2 = MultiLayerPagedKVCache4Bit(64, 16, kvlen + 256, "cuda", 1, nkv, d, dtype=torch.bfloat16)
         cache2.update(kv[0][:, :, :kvlen].transpose(1, 2).contiguous(), kv[1][:, :, :kvlen].transpose(1, 2).contiguous(), 0)
         step = layers.GraphedDecodeStep(layer, cache2, 64, hidden)
         step.x.copy_(x)                       # the layer's input sits in the graph's input buffer, as the
         ms_g = timed(lambda: step(step.x))    # previous layer's output would; the bf16 layer reads x in place too
-        rows.append({"config": f"decoder layer decode batch 64, KV length {kvlen}+, INT4 paged KV cache, HIP graph",
-                     "fmt": fmt, "arc_ms": round(ms_g, 3), "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_g, 2),
-                     "tokens_per_s": round(64 / ms_g * 1e3)})
+        rows.append({"config": f"decoder layer decode batch 64, KV length {kvlen}+, both steps as HIP graphs "
+                               f"(ARC: INT4 paged KV cache; bf16: bf16 KV cache + SDPA)",
+                     "fmt": fmt, "arc_ms": round(ms_g, 3), "bf16_ms": round(ms_bf_graph, 3),
+                     "speedup": round(ms_bf_graph / ms_g, 2), "tokens_per_s": round(64 / ms_g * 1e3)})
         print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
-        del layer, W, kv, x, cache, cache2, step
+        del layer, W, kv, x, cache, cache2, step, bf_graph
         torch.cuda.empty_cache()
 
-    # Mixtral block (benchmark configuration 5: NVFP4; MXFP4 beside it), select_num 128
+    # Mixtral block (benchmark configuration 5: NVFP4; MXFP4 beside it), select_num 128, per-expert channel
+    # orders from the per-expert channel maxima of the routed tokens
     E, ffn, tokens = 8, 14336, 4096
     g = torch.Generator().manual_seed(5)
-    x = torch.randn(1, tokens, hidden, generator=g).to(torch.bfloat16).cuda()
+    xcpu = recipes.activations(tokens, hidden, seed=5, outlier_frac=0.01, outlier_gain=40.0)
+    x = xcpu.cuda().view(1, tokens, hidden)
     bias = torch.log(1.0 / torch.arange(1, E + 1).float() ** 1.1)
-    logits = (torch.randn(tokens, E, generator=g) + bias).cuda()
+    logits_cpu = torch.randn(tokens, E, generator=g) + bias
+    logits = logits_cpu.cuda()
+    sel = torch.topk(F.softmax(logits_cpu, dim=1), 2, dim=-1)[1]
+    indices = []
+    for e in range(E):
+        mine = xcpu[(sel == e).any(1)]
+        indices.append((recipes.reorder_index(mine if mine.numel() else xcpu).cuda(),
+                        torch.randperm(ffn, generator=g).to(torch.int16).cuda()))
     moe_ms = {}
     for fmt in ("NVFP4", "MXFP4"):
-        block = layers.build_mixtral_block(hidden, ffn, E, 2, 128, fmt, seed=5)
-        moe_ms[fmt] = timed(lambda: block(x, router_logits=logits))
+        block = layers.build_mixtral_block(hidden, ffn, E, 2, 128, fmt, indices=indices, seed=5)
+        grouped = timed(lambda: block(x, router_logits=logits))
+        block.grouped = False
+        moe_ms[fmt] = (grouped, timed(lambda: block(x, router_logits=logits)))
         del block
         torch.cuda.empty_cache()
     # the same block in bf16 on dequantised-size weights (random: only the time matters)
@@ -289,9 +355,10 @@ def layer_rows(torch, iters=10):
         return out
 
     ms_bf = timed(bf16_moe)
-    counts = torch.bincount(torch.topk(F.softmax(logits, dim=1), 2, dim=-1)[1].reshape(-1), minlength=E).tolist()
-    for fmt, ms_arc in moe_ms.items():
-        rows.append({"config": "Mixtral MoE block, 4096 tokens, 8 experts top-2", "fmt": fmt, "arc_ms": round(ms_arc, 3),
+    counts = torch.bincount(sel.reshape(-1), minlength=E).tolist()
+    for fmt, (ms_arc, ms_loop) in moe_ms.items():
+        rows.append({"config": "Mixtral MoE block, 4096 tokens, 8 experts top-2, grouped launches", "fmt": fmt,
+                     "arc_ms": round(ms_arc, 3), "arc_per_expert_loop_ms": round(ms_loop, 3),
                      "bf16_ms": round(ms_bf, 3), "speedup": round(ms_bf / ms_arc, 2), "tokens_per_expert": counts,
                      "tokens_per_s": round(tokens / ms_arc * 1e3)})
         print("[bench] layer", json.dumps(rows[-1]), file=sys.stderr, flush=True)
@@ -303,9 +370,16 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--gemm-table", action="store_true", help="every benchmark GEMM shape x M (slower)")
+    ap.add_argument("--quick", action="store_true", help="no layer rows, two GEMM shapes")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="the headline kernel and the copy kernels only (what a counter run should see)")
+    ap.add_argument("--gemm-table", action="store_true", help="(kept for older command lines: the full table is the default)")
+    ap.add_argument("--layers", action="store_true", help="(kept for older command lines: the layer rows are the default)")
     ap.add_argument("--no-gemm", action="store_true")
-    ap.add_argument("--layers", action="store_true", help="also time a decoder layer and an MoE block (configs 4, 5)")
+    ap.add_argument("--no-quantize-table", action="store_true")
+    ap.add_argument("--gemm-shapes", default="", help="NxK[,NxK...]: restrict the GEMM rows to these shapes (counter runs)")
+    ap.add_argument("--gemm-ms", default="", help="M[,M...]: restrict the GEMM rows to these M")
+    ap.add_argument("--no-layers", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=M_TOKENS)
     args = ap.parse_args()
@@ -331,13 +405,13 @@ def main():
     nbuf = max(2, int(1.2e9 // bytes_per_launch))          # ~1.2 GB of rotating traffic
     base = recipes.activations(M_TOKENS, H, seed=2, outlier_frac=0.005, outlier_gain=50.0)
     gam = recipes.gamma(H, seed=7).cuda()
-    idx = recipes.reorder_index(base).cuda()               # any permutation gives the same traffic
+    idx = recipes.reorder_index(base).cuda()               # ascending per-channel maxima, as the reference calibrates
     xs = [base.cuda() if i == 0 else (base.cuda().roll(i, 0)) for i in range(nbuf)]
     fid = {"NVFP4": 0, "MXFP4": 1}
 
-    def outputs(fmt, S):
-        return (torch.empty(L.arcq_codes_bytes(M_TOKENS, H, S), dtype=torch.uint8, device="cuda"),
-                torch.empty(L.arcq_scales_bytes(M_TOKENS, H, S, fid[fmt]), dtype=torch.uint8, device="cuda"))
+    def outputs(fmt, S, rows=M_TOKENS):
+        return (torch.empty(L.arcq_codes_bytes(rows, H, S), dtype=torch.uint8, device="cuda"),
+                torch.empty(L.arcq_scales_bytes(rows, H, S, fid[fmt]), dtype=torch.uint8, device="cuda"))
 
     outs = [outputs(FMT, SELECT) for _ in range(nbuf)]
     torch.cuda.synchronize()
@@ -367,51 +441,35 @@ def main():
     # ---------------- roofline of the dominant kernel: HIP events over the same timed region ----------------
     kern_ms = ev0.elapsed_time(ev1) / args.steps           # launches are queued back to back: GPU time per launch
     achieved = bytes_per_launch / (kern_ms * 1e-3) / 1e9
-    # the box's own streaming ceiling for this read:write mix (plain copy kernel, same bytes)
+    # the box's own streaming ceiling for this read:write mix: plain copy kernels moving the same bytes, in every
+    # launch shape the library has (loads in flight per thread, non-temporal, resident / one-round grids, LDS-direct)
     b_in = M_TOKENS * H * 2
     b_out = ((bytes_per_launch - b_in) // 16) * 16
     sdst = [torch.empty(b_out, dtype=torch.uint8, device="cuda") for _ in range(nbuf)]
-
-    def probe(i):
-        L.arcq_stream_probe(xs[i % nbuf].data_ptr(), sdst[i % nbuf].data_ptr(), b_in, b_out, stream)
-
-    for i in range(10):
-        probe(i)
-    probe_ms = loop_time_ms(probe, 100, torch)
+    probes = {}
+    for variant in range(L.arcq_stream_probe_variants()):
+        def probe(i, variant=variant):
+            L.arcq_stream_probe_variant(xs[i % nbuf].data_ptr(), sdst[i % nbuf].data_ptr(), b_in, b_out, variant, stream)
+        for i in range(10):
+            probe(i)
+        probes[variant] = loop_time_ms(probe, 100, torch)
+    best_variant = min(probes, key=probes.get)
+    probe_ms = probes[best_variant]
     ceiling = (b_in + b_out) / probe_ms / 1e6
-    roofline = {"bound": "hbm", "kernel": "quantize_rows_unit_kernel<NVFP4, RMSNORM>", "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+    workload_key = f"fused-norm {FMT} M={M_TOKENS} K={H} S={SELECT}"
+    traffic, traffic_kernel, traffic_source = measured_traffic(workload_key)
+    roofline = {"bound": "hbm", "kernel": "quantize_rows_wave_kernel<NVFP4, RMSNORM, K/1024 = 4>", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "traffic_source": traffic_source, "traffic_kernel": traffic_kernel,
                 "bytes_per_launch": bytes_per_launch, "avg_launch_us": round(kern_ms * 1e3, 2),
                 "streaming_copy_same_bytes": {"us": round(probe_ms * 1e3, 2), "GB/s": round(ceiling, 1),
-                                              "frac_of_peak": round(ceiling / HBM_PEAK_GBS, 4)},
+                                              "frac_of_peak": round(ceiling / HBM_PEAK_GBS, 4), "variant": best_variant,
+                                              "all_variants_us": {str(k): round(v * 1e3, 2) for k, v in probes.items()}},
+                "frac_of_streaming_copy": round(probe_ms / kern_ms, 4),
                 "note": "algorithmic bytes / (HIP-event time over the timed region / launches); "
-                        "streaming_copy_same_bytes is a plain copy kernel moving the same bytes on this box; "
-                        "traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/)"}
-
-    # ---------------- other quantize configurations (reported, not the headline) ----------------
-    others = {}
-    # the NVFP4 tensor scale the reference's callers compute: max|x| / (448 * 6) (model/qLlamaLayer.py:74)
-    gs_dev = (xs[0].abs().max().float() / 2688.0).reshape(())
-    for fmt, S, kind in (("MXFP4", 256, "norm"), ("NVFP4", 64, "norm"), ("NVFP4", 256, "x_unit"), ("MXFP4", 256, "x_unit"),
-                         ("NVFP4", 256, "x_scaled")):
-        q, sf = outputs(fmt, S)
-        if kind == "norm":
-            fn = lambda i, fmt=fmt, S=S, q=q, sf=sf: L.arcq_rmsnorm_quantize_x(
-                xs[i % nbuf].data_ptr(), gam.data_ptr(), EPS, M_TOKENS, H, idx.data_ptr(), S, fid[fmt], 1.0, None,
-                q.data_ptr(), sf.data_ptr(), stream)
-        else:
-            dgs = ctypes.c_void_p(gs_dev.data_ptr()) if kind == "x_scaled" else None
-            fn = lambda i, fmt=fmt, S=S, q=q, sf=sf, dgs=dgs: L.arcq_reorder_quantize_x(
-                xs[i % nbuf].data_ptr(), M_TOKENS, H, idx.data_ptr(), S, fid[fmt], 1.0, dgs, q.data_ptr(), sf.data_ptr(),
-                stream)
-        for i in range(5):
-            fn(i)
-        ms = loop_time_ms(fn, 100, torch)
-        b = quant_bytes(M_TOKENS, H, S, fmt, kind == "norm")
-        name = {"norm": "rmsnorm_quantize_x", "x_unit": "reorder_quantize_x(scale=1)",
-                "x_scaled": "reorder_quantize_x(device tensor scale)"}[kind]
-        others[f"{name}/{fmt}/S{S}"] = {"us": round(ms * 1e3, 2), "GB/s": round(b / ms / 1e6, 1),
-                                        "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)}
+                        "streaming_copy_same_bytes is the fastest of the library's plain copy kernels moving the same "
+                        "bytes on this box (a 44 MB launch cannot reach the peak: the copy shows what one can); "
+                        "traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (traffic_source)"}
 
     out = {
         "metric": "ARC FP4 GEMM TFLOPS + quantize GB/s at Llama-3-8B shapes, M=1..4096",
@@ -423,17 +481,57 @@ def main():
                                f"C-ABI call; value = algorithmic bytes / wall time; inputs rotate over {nbuf} "
                                f"buffers ({nbuf * bytes_per_launch / 1e9:.2f} GB) to defeat the 256 MB Infinity Cache"},
         "roofline": roofline,
-        "quantize_other": others,
     }
+    if args.headline_only:
+        print(json.dumps(out), flush=True)
+        return
+
+    # ---------------- benchmark configuration 2 in full, and the plain quantizers (reported, not the headline) ----------------
+    def time_quant(fn, rows, reps):
+        for i in range(5):
+            fn(i)
+        return loop_time_ms(fn, reps, torch)
+
+    quant = []
+    # the NVFP4 tensor scale the reference's callers compute: max|x| / (448 * 6) (model/qLlamaLayer.py:74)
+    gs_dev = (xs[0].abs().max().float() / 2688.0).reshape(())
+    for fmt in (() if args.no_quantize_table else ("NVFP4", "MXFP4")):
+        for S in (64, 256):
+            for rows in (1, 16, 256, 4096):
+                q, sf = outputs(fmt, S, rows)
+                fn = lambda i, fmt=fmt, S=S, q=q, sf=sf, rows=rows: L.arcq_rmsnorm_quantize_x(
+                    xs[i % nbuf].data_ptr(), gam.data_ptr(), EPS, rows, H, idx.data_ptr(), S, fid[fmt], 1.0, None,
+                    q.data_ptr(), sf.data_ptr(), stream)
+                ms = time_quant(fn, rows, 100)
+                b = quant_bytes(rows, H, S, fmt, True)
+                quant.append({"op": "rmsnorm_quantize_x", "fmt": fmt, "select_num": S, "M": rows, "us": round(ms * 1e3, 2),
+                              "GB/s": round(b / ms / 1e6, 1), "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)})
+    for fmt, S, kind in (() if args.no_quantize_table else
+                         (("NVFP4", 256, "x_unit"), ("MXFP4", 256, "x_unit"), ("NVFP4", 256, "x_scaled"))):
+        q, sf = outputs(fmt, S)
+        dgs = ctypes.c_void_p(gs_dev.data_ptr()) if kind == "x_scaled" else None
+        fn = lambda i, fmt=fmt, S=S, q=q, sf=sf, dgs=dgs: L.arcq_reorder_quantize_x(
+            xs[i % nbuf].data_ptr(), M_TOKENS, H, idx.data_ptr(), S, fid[fmt], 1.0, dgs, q.data_ptr(), sf.data_ptr(),
+            stream)
+        ms = time_quant(fn, M_TOKENS, 100)
+        b = quant_bytes(M_TOKENS, H, S, fmt, False)
+        name = {"x_unit": "reorder_quantize_x (tensor scale 1)", "x_scaled": "reorder_quantize_x (tensor scale max|x|/2688 on the device)"}[kind]
+        quant.append({"op": name, "fmt": fmt, "select_num": S, "M": M_TOKENS, "us": round(ms * 1e3, 2),
+                      "GB/s": round(b / ms / 1e6, 1), "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)})
+    out["quantize"] = quant
+    del xs[1:], outs[1:], sdst[1:]
+    torch.cuda.empty_cache()
 
     if not args.no_gemm:
-        # default: the qkv and gate_up projections of Llama-3-8B (the smallest and the largest weight of a layer)
-        shapes = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)] if args.gemm_table else \
-            [(6144, 4096), (28672, 4096)]
-        Ms = [1, 16, 64, 128, 512, 2048, 4096] if args.gemm_table else [1, 16, 64, 512, 4096]
+        shapes = [(6144, 4096), (28672, 4096)] if args.quick else [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]
+        Ms = [1, 16, 128, 512, 2048, 4096]                  # benchmark configuration 3
+        if args.gemm_shapes:
+            shapes = [tuple(int(v) for v in t.split("x")) for t in args.gemm_shapes.split(",")]
+        if args.gemm_ms:
+            Ms = [int(v) for v in args.gemm_ms.split(",")]
         out["gemm"] = gemm_rows(torch, agemm, shapes, Ms, ["MXFP4", "NVFP4"])
         out["gemm_peaks_tflops"] = MFMA_PEAK_TFLOPS
-    if args.layers:
+    if not (args.quick or args.no_layers):
         out["layers"] = layer_rows(torch)
 
     if not args.no_cpu:
