@@ -1135,7 +1135,12 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
     return plan;
   }
   if (fmt == ARCQ_FMT_NVFP4 && force != 0 && tiled_ok) {
-    plan.kernel = force > 1 ? force : (M > 1024 ? 44 : (M > 128 && !one_round_21 ? 22 : 21));
+    // 256x256 tiles where they fill at least three quarters of the CUs (they decode each operand row for the
+    // fewest MFMAs); with fewer of them half the machine idles (4096 x 4096 at M = 2048: 128 tiles, 105 us
+    // against 74 us with 256x128 tiles), so the next smaller tile that still fills it
+    const long t44 = (long)((M + 255) / 256) * ((N + 255) / 256), t42 = (long)((M + 127) / 128) * ((N + 255) / 256);
+    const int pick = t44 >= 192 ? 44 : (M > 128 && !one_round_21 ? (t42 >= 192 ? 42 : 22) : 21);
+    plan.kernel = force > 1 ? force : pick;
     return plan;
   }
   plan.kernel = 0;
