@@ -73,6 +73,11 @@ def lib() -> ctypes.CDLL:
     L.arcq_grouped_swiglu_quantize_x.argtypes = [vp, vp, i, i, i, vp, i, vp, i, i, vp, vp, vp, vp]
     L.arcq_grouped_tensor_scale.argtypes = [vp, vp, i, i, i, vp, i, f, vp, vp]
     L.arcq_grouped_matmul.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, f, vp, vp, vp, vp, vp]
+    L.arcq_grouped_matmul_swiglu.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i, f, vp, vp, vp, vp, vp]
+    L.arcq_matmul_swiglu.argtypes = [vp, vp, vp, vp, i, i, i, i, f, vp, vp, vp, vp, vp]
+    L.arcq_scales_from_absmax.argtypes = [vp, i, f, vp]
+    for name in ("arcq_grouped_matmul_swiglu", "arcq_matmul_swiglu", "arcq_scales_from_absmax"):
+        getattr(L, name).restype = i
     L.arcq_moe_combine.argtypes = [vp, vp, vp, i, i, i, i, vp, vp]
     L.arcq_moe_combine.restype = i
     for name in ("arcq_grouped_reorder_quantize_x", "arcq_grouped_swiglu_quantize_x", "arcq_grouped_tensor_scale",

@@ -33,7 +33,8 @@ from ._lib import FORMATS, ArcqError  # noqa: F401
 __all__ = ["matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "init_kv_i4", "append_kv_i4",
            "batch_decode_i4", "swiglu_quantize_x", "tensor_scale", "prepare_stream", "dequantize", "check_index",
            "unpack_codes", "scale_values", "grouped_tensor_scale", "grouped_reorder_quantize_x",
-           "grouped_swiglu_quantize_x", "grouped_matmul", "moe_combine"]
+           "grouped_swiglu_quantize_x", "grouped_matmul", "moe_combine", "matmul_swiglu",
+           "grouped_matmul_swiglu", "interleave_gate_up"]
 
 
 def _fmt_id(fmt) -> int:
@@ -373,6 +374,96 @@ def grouped_matmul(A, B, SFA, SFB, seg, scale_a=None, scale_b=None, *, fmt=None,
                                             None if residual is None else residual.data_ptr(), C.data_ptr(), _stream(A))
     _lib.check(rc, "arcq_grouped_matmul")
     return C
+
+
+def interleave_gate_up(w_gate, w_up):
+    """[F, K] gate and up weights -> [2F, K] with rows gate_0, up_0, gate_1, up_1, ...: the row order the
+    SwiGLU-fused GEMMs expect (quantize the result with reorder_quantize_w as usual)."""
+    if w_gate.shape != w_up.shape:
+        raise RuntimeError("gate and up weights must have the same shape")
+    return torch.stack((w_gate, w_up), dim=1).reshape(2 * w_gate.shape[0], w_gate.shape[1]).contiguous()
+
+
+def _absmax_to_scales(buf, divisor):
+    with _on_device(buf):
+        _lib.check(_lib.lib().arcq_scales_from_absmax(buf.data_ptr(), buf.numel(), float(divisor), _stream(buf)),
+                   "arcq_scales_from_absmax")
+    return buf
+
+
+def matmul_swiglu(A, B, SFA, SFB, scale, *, fmt=None, tensor_scale=False):
+    """matmul for a fused gate/up projection whose weight rows alternate gate, up (interleave_gate_up), with
+    act_fn(gate) * up formed in the epilogue: returns t bf16 [M, N/2], bit-identical to
+    ``h = matmul(...); F.silu(h_gate) * h_up`` in bf16, without h going through memory.  tensor_scale=True
+    also returns the NVFP4 tensor scale max|t| / 2688 of t (0-dim fp32 device tensor, 1 for all zeros)."""
+    _require(A, "A", torch.uint8, 2)
+    _require(B, "B", torch.uint8, 2)
+    _require(SFA, "SFA", torch.uint8)
+    _require(SFB, "SFB", torch.uint8)
+    if A.shape[1] != B.shape[1]:
+        raise RuntimeError(f"A and B disagree on K': {2 * A.shape[1]} vs {2 * B.shape[1]}")
+    f = _infer_fmt(A, SFA, fmt)
+    M, N, Kp = A.shape[0], B.shape[0], 2 * A.shape[1]
+    G = _lib.GROUP_SIZE[f]
+    if SFA.numel() != M * (Kp // G) or SFB.numel() != N * (Kp // G):
+        raise RuntimeError("scale buffers do not match the code buffers")
+    if Kp % 128 or Kp < 512 or N % 16:
+        raise RuntimeError(f"Value error in matmul_swiglu: K'={Kp} (multiple of 128, >= 512), N={N} (multiple of 16)")
+    if isinstance(scale, (tuple, list)):
+        ha, da, ka = _scalar(scale[0], A.device)
+        hb, db, kb = _scalar(scale[1], A.device)
+        alpha = ha * hb
+    else:
+        alpha, da, ka = _scalar(scale, A.device)
+        db, kb = None, None
+    T = torch.empty((M, N // 2), dtype=torch.bfloat16, device=A.device)
+    amax = torch.zeros(1, dtype=torch.float32, device=A.device) if tensor_scale else None
+    with _on_device(A):
+        rc = _lib.lib().arcq_matmul_swiglu(A.data_ptr(), SFA.data_ptr(), B.data_ptr(), SFB.data_ptr(), M, N, Kp, f, alpha,
+                                           da, db, T.data_ptr(), None if amax is None else amax.data_ptr(), _stream(A))
+    _lib.check(rc, "arcq_matmul_swiglu")
+    del ka, kb
+    if tensor_scale:
+        return T, _absmax_to_scales(amax, 2688.0).reshape(())
+    return T
+
+
+def grouped_matmul_swiglu(A, B, SFA, SFB, seg, scale_a=None, scale_b=None, *, fmt=None, tensor_scale=False):
+    """grouped_matmul with the SwiGLU epilogue of matmul_swiglu (B[e] rows alternate gate, up): t bf16 [M, N/2];
+    tensor_scale=True also returns the per-expert NVFP4 tensor scales max|t_e| / 2688 as fp32 [E]."""
+    _require(A, "A", torch.uint8, 2)
+    _require(B, "B", torch.uint8, 3)
+    _require(SFA, "SFA", torch.uint8)
+    _require(SFB, "SFB", torch.uint8)
+    E = _seg(seg, A.device)
+    if B.shape[0] != E or A.shape[1] != B.shape[2]:
+        raise RuntimeError(f"B must be [{E}, N, {A.shape[1]}]")
+    f = _infer_fmt(A, SFA, fmt)
+    M, N, Kp = A.shape[0], B.shape[1], 2 * A.shape[1]
+    G = _lib.GROUP_SIZE[f]
+    if SFA.numel() != M * (Kp // G) or SFB.numel() != E * N * (Kp // G):
+        raise RuntimeError("scale buffers do not match the code buffers")
+    if Kp % 128 or Kp < 512 or N % 16:
+        raise RuntimeError(f"Value error in grouped_matmul_swiglu: K'={Kp}, N={N}")
+    ptrs = []
+    for t, name in ((scale_a, "scale_a"), (scale_b, "scale_b")):
+        if t is None:
+            ptrs.append(None)
+            continue
+        _require(t, name, torch.float32, 1)
+        if t.numel() != E or t.device != A.device:
+            raise RuntimeError(f"{name} must be fp32 [{E}] on A's device")
+        ptrs.append(t.data_ptr())
+    T = torch.empty((M, N // 2), dtype=torch.bfloat16, device=A.device)
+    amax = torch.zeros(E, dtype=torch.float32, device=A.device) if tensor_scale else None
+    with _on_device(A):
+        rc = _lib.lib().arcq_grouped_matmul_swiglu(A.data_ptr(), SFA.data_ptr(), B.data_ptr(), SFB.data_ptr(),
+                                                   seg.data_ptr(), E, M, N, Kp, f, 1.0, ptrs[0], ptrs[1], T.data_ptr(),
+                                                   None if amax is None else amax.data_ptr(), _stream(A))
+    _lib.check(rc, "arcq_grouped_matmul_swiglu")
+    if tensor_scale:
+        return T, _absmax_to_scales(amax, 2688.0)
+    return T
 
 
 def moe_combine(y, position, weight, tokens, top_k):

@@ -44,7 +44,7 @@ def _stale(target: str, deps) -> bool:
 
 def build_hip(force: bool = False, verbose: bool = False) -> str:
     srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
-    deps = srcs + [os.path.join(CSRC, h) for h in ("arcq_math.h", "arcq_internal.h")] + [
+    deps = srcs + [os.path.join(CSRC, h) for h in ("arcq_math.h", "arcq_internal.h", "arcq_swiglu.h")] + [
         os.path.join(HERE, "..", "include", "arcq.h")]
     if force or _stale(HIP_LIB, deps):
         cmd = [_hipcc(), *HIPCC_FLAGS, "-o", HIP_LIB, *srcs]

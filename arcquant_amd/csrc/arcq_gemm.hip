@@ -18,6 +18,7 @@
 
 #include "arcq_internal.h"
 #include "arcq_math.h"
+#include "arcq_swiglu.h"
 
 namespace arcq {
 namespace {
@@ -47,6 +48,14 @@ struct GemmParams {
   const int *seg = nullptr;
   int n_seg = 0;
   size_t seg_b_codes = 0, seg_b_scales = 0;
+  // fused SwiGLU epilogue (tiled kernels): the weight rows alternate gate, up, gate, up ..., so that output
+  // columns 2j and 2j+1 are gate_j and up_j of one token and sit in one lane; c then is bf16 [M, N/2] and
+  // receives act_fn(gate) * up formed from the bf16-rounded GEMM outputs, exactly what the unfused sequence
+  // (GEMM, then silu and multiply in bf16) gives.  absmax_bits: NULL, or one word per segment (one word when
+  // not grouped) that collects max |output| as the bits of a non-negative float (zeroed by the caller).
+  int swiglu = 0;
+  uint32_t *absmax_bits = nullptr;
+  int seg_index = 0;
 };
 
 // Grouped launches: maps the workgroup to (segment, tile) and turns p into that segment's problem (M = its
@@ -68,13 +77,14 @@ __device__ __forceinline__ bool enter_segment(GemmParams &p, int &lin) {
       const size_t kbytes = p.Kp >> 1, ksc = p.Kp / G;
       p.a_codes += (size_t)beg * kbytes;
       p.a_scales += (size_t)beg * ksc;
-      p.c += (size_t)beg * p.N;
+      p.c += (size_t)beg * (p.swiglu ? p.N >> 1 : p.N);
       if (p.residual) p.residual += (size_t)beg * p.N;
       p.b_codes += (size_t)e * p.seg_b_codes;
       p.b_scales += (size_t)e * p.seg_b_scales;
       if (p.d_alpha_a) p.d_alpha_a += e;
       if (p.d_alpha_b) p.d_alpha_b += e;
       p.M = cnt;
+      p.seg_index = e;
       return true;
     }
     lin -= t;
@@ -301,6 +311,10 @@ __device__ __forceinline__ void wait_dma_and_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+template <int WN, int WM>
+__device__ __forceinline__ void store_workgroup_tile_swiglu_fwd(const GemmParams &p, v16f (&acc)[WN][WM], uint8_t *ldsA,
+                                                                uint8_t *ldsB, int m_base, int n_base, int wave, int lane);
+
 // Epilogue shared by the tiled kernels: acc[i][j] is the 32x32 tile (n-tile i, m-tile j) of the
 // wave tile.  ldsA / ldsB: two LDS areas of at least 2*32*WM*64*WN bytes each, free for reuse.
 template <int WN, int WM>
@@ -309,6 +323,7 @@ __device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (
   constexpr int BN = 64 * WN, BM = 64 * WM;
   const int r = lane & 31, kh = lane >> 5;
   const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;
+  if (p.swiglu) return store_workgroup_tile_swiglu_fwd<WN, WM>(p, acc, ldsA, ldsB, m_base, n_base, wave, lane);
   if (p.partial) {  // split-K: the unscaled fp32 tile of this K range
     float *part = p.partial + (size_t)blockIdx.y * p.M * p.N;
 #pragma unroll
@@ -379,6 +394,90 @@ __device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (
 #pragma unroll
     for (int j = 0; j < WM; ++j)
       store_tile(p, acc[i][j], m_base + wm0 + 32 * j, n_base + wn0 + 32 * i, lane, alpha);
+}
+
+// Fused SwiGLU epilogue of the tiled kernels (p.swiglu): a lane's four consecutive columns of one row are
+// (gate_j, up_j, gate_j+1, up_j+1); each is rounded to bf16 as the plain epilogue would store it, and the two
+// products act_fn(gate) * up leave as one dword.  Whole tiles go through LDS so that every store
+// instruction writes 16 bytes per lane along output rows; ragged tiles store dwords with bounds checks.
+template <int WN, int WM>
+__device__ __forceinline__ void store_workgroup_tile_swiglu(const GemmParams &p, v16f (&acc)[WN][WM], uint8_t *ldsA,
+                                                            uint8_t *ldsB, int m_base, int n_base, int wave, int lane) {
+  constexpr int BN = 64 * WN, BM = 64 * WM;
+  const int r = lane & 31, kh = lane >> 5;
+  const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;
+  const float alpha = effective_alpha(p);
+  const int No = p.N >> 1;  // output columns
+  uint32_t amax = 0u;       // max |t| of this lane as bf16 bits without the sign
+  auto product = [&](const v16f &a, int q) {  // the hardware's RNE convert: the bits f32_to_bf16_bits gives
+    return swiglu_pair(pack_bf16_rne(a[4 * q] * alpha, a[4 * q + 2] * alpha),
+                       pack_bf16_rne(a[4 * q + 1] * alpha, a[4 * q + 3] * alpha));
+  };
+  auto track = [&](uint32_t t) {
+    const uint32_t lo = t & 0x7fffu, hi = (t >> 16) & 0x7fffu;
+    amax = lo > amax ? lo : amax;
+    amax = hi > amax ? hi : amax;
+  };
+  constexpr bool kPow2 = (WN & (WN - 1)) == 0;
+  if (kPow2 && m_base + BM <= p.M && n_base + BN <= p.N && (No & 7) == 0) {
+    wait_dma_and_sync();  // every wave is done reading operands
+    constexpr int RB = 32 * WN;   // bytes per row of the wave tile: 16 * WN products
+    constexpr int LPR = 2 * WN;   // lanes per row when reading 16 bytes each
+    uint8_t *region = (wave < 2 ? ldsA : ldsB) + (wave & 1) * (32 * WM * RB);
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
+#pragma unroll
+      for (int j = 0; j < WM; ++j) {
+        const int m = 32 * j + r;
+        const int sw = m & (LPR - 1);                 // swizzle of the row's 16-byte groups
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t t = product(acc[i][j], q);
+          track(t);
+          const int c = 8 * i + 2 * q + kh;           // dword of the row
+          *reinterpret_cast<uint32_t *>(region + m * RB + ((((c >> 2) ^ sw) << 2) | (c & 3)) * 4) = t;
+        }
+      }
+    const int rr = lane / LPR, tq = lane % LPR;
+    uint16_t *cbase = p.c + (size_t)(m_base + wm0) * No + ((n_base + wn0) >> 1) + 8 * tq;
+#pragma unroll
+    for (int it = 0; it < (32 * WM * LPR) / 64; ++it) {
+      const int m = it * (64 / LPR) + rr;
+      const int sw = m & (LPR - 1);
+      const uint4 v = *reinterpret_cast<const uint4 *>(region + m * RB + ((tq ^ sw) << 4));
+      *reinterpret_cast<uint4 *>(cbase + (size_t)m * No) = v;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
+#pragma unroll
+      for (int j = 0; j < WM; ++j) {
+        const int m = m_base + wm0 + 32 * j + r;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n_base + wn0 + 32 * i + 8 * q + 4 * kh;
+          const uint32_t t = product(acc[i][j], q);   // every lane computes (the special-value test of the
+          if (m < p.M && n + 3 < p.N) {               // activation function is a vote of the whole wave)
+            track(t);
+            *reinterpret_cast<uint32_t *>(p.c + (size_t)m * No + (n >> 1)) = t;
+          }
+        }
+      }
+  }
+  if (p.absmax_bits) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t v = (uint32_t)__shfl_xor((int)amax, o);
+      amax = v > amax ? v : amax;
+    }
+    if (lane == 0 && amax) atomicMax(p.absmax_bits + p.seg_index, amax << 16);  // bf16 bits -> fp32 bits
+  }
+}
+
+template <int WN, int WM>
+__device__ __forceinline__ void store_workgroup_tile_swiglu_fwd(const GemmParams &p, v16f (&acc)[WN][WM], uint8_t *ldsA,
+                                                                uint8_t *ldsB, int m_base, int n_base, int wave, int lane) {
+  store_workgroup_tile_swiglu<WN, WM>(p, acc, ldsA, ldsB, m_base, n_base, wave, lane);
 }
 
 // An FP4 operand of the scaled MFMA is 4 registers; the builtin's type has 8, the upper 4 unused.
@@ -1322,16 +1421,19 @@ extern "C" int arcq_matmul_add(const void *a_codes, const void *a_scales, const 
                            stream);
 }
 
-extern "C" int arcq_grouped_matmul(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
-                                   const int *seg_offsets, int n_seg, int M, int N, int Kp, int fmt, float alpha,
-                                   const float *d_alpha_a, const float *d_alpha_b, const void *residual, void *c,
-                                   void *stream) {
-  using namespace arcq;
+namespace arcq {
+namespace {
+
+int grouped_matmul_impl(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                        const int *seg_offsets, int n_seg, int M, int N, int Kp, int fmt, float alpha,
+                        const float *d_alpha_a, const float *d_alpha_b, const void *residual, void *c, bool swiglu,
+                        float *d_absmax, void *stream) {
   GemmParams p;
   const int rc = check_gemm_args(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b,
                                  residual, c, &p);
   if (rc != ARCQ_OK || M == 0 || N == 0) return rc;
   if (n_seg < 1 || Kp % 128 != 0 || Kp < 512) return ARCQ_ERR_SHAPE;  // the tiled kernels' shapes only
+  if (swiglu && (N % 16 != 0 || residual)) return ARCQ_ERR_SHAPE;
   if (!seg_offsets) return ARCQ_ERR_NULL;
   if (!aligned16(a_scales) || !aligned16(b_scales) || (residual && !aligned16(residual))) return ARCQ_ERR_ALIGN;
   const int G = fmt == ARCQ_FMT_NVFP4 ? 16 : 32;
@@ -1339,6 +1441,8 @@ extern "C" int arcq_grouped_matmul(const void *a_codes, const void *a_scales, co
   p.n_seg = n_seg;
   p.seg_b_codes = (size_t)N * (Kp >> 1);
   p.seg_b_scales = (size_t)N * (Kp / G);
+  p.swiglu = swiglu ? 1 : 0;
+  p.absmax_bits = reinterpret_cast<uint32_t *>(d_absmax);
   // Tile from the rows an average segment holds (the real counts live on the device).  The larger tiles are
   // faster per flop, but every segment ends in a partly empty tile of rows and skewed routing leaves some
   // segments far below the average: on 8192 rows over 8 segments of 195..3120 rows the 128x128 tile beat
@@ -1349,4 +1453,62 @@ extern "C" int arcq_grouped_matmul(const void *a_codes, const void *a_scales, co
   plan.kernel = avg >= 2048 ? 44 : (avg >= 96 ? 22 : 21);
   if (force == 44 || force == 42 || force == 22 || force == 21) plan.kernel = force;
   return run_gemm(p, plan, fmt, nullptr, static_cast<hipStream_t>(stream));
+}
+
+__global__ void scales_from_absmax_kernel(float *v, int n, float divisor) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float scale = v[i] / divisor;
+  v[i] = scale == 0.0f ? 1.0f : scale;
+}
+
+}  // namespace
+}  // namespace arcq
+
+extern "C" int arcq_grouped_matmul(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                                   const int *seg_offsets, int n_seg, int M, int N, int Kp, int fmt, float alpha,
+                                   const float *d_alpha_a, const float *d_alpha_b, const void *residual, void *c,
+                                   void *stream) {
+  return arcq::grouped_matmul_impl(a_codes, a_scales, b_codes, b_scales, seg_offsets, n_seg, M, N, Kp, fmt, alpha,
+                                   d_alpha_a, d_alpha_b, residual, c, false, nullptr, stream);
+}
+
+extern "C" int arcq_grouped_matmul_swiglu(const void *a_codes, const void *a_scales, const void *b_codes,
+                                          const void *b_scales, const int *seg_offsets, int n_seg, int M, int N, int Kp,
+                                          int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b, void *t,
+                                          float *d_absmax, void *stream) {
+  return arcq::grouped_matmul_impl(a_codes, a_scales, b_codes, b_scales, seg_offsets, n_seg, M, N, Kp, fmt, alpha,
+                                   d_alpha_a, d_alpha_b, nullptr, t, true, d_absmax, stream);
+}
+
+extern "C" int arcq_matmul_swiglu(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                                  int M, int N, int Kp, int fmt, float alpha, const float *d_alpha_a,
+                                  const float *d_alpha_b, void *t, float *d_absmax, void *stream) {
+  using namespace arcq;
+  GemmParams p;
+  const int rc = check_gemm_args(a_codes, a_scales, b_codes, b_scales, M, N, Kp, fmt, alpha, d_alpha_a, d_alpha_b,
+                                 nullptr, t, &p);
+  if (rc != ARCQ_OK || M == 0 || N == 0) return rc;
+  if (Kp % 128 != 0 || Kp < 512 || N % 16 != 0) return ARCQ_ERR_SHAPE;  // the tiled kernels' shapes only
+  if (!aligned16(a_scales) || !aligned16(b_scales)) return ARCQ_ERR_ALIGN;
+  p.swiglu = 1;
+  p.absmax_bits = reinterpret_cast<uint32_t *>(d_absmax);
+  GemmPlan plan = plan_gemm(M, N, Kp, fmt, true);
+  const bool tiled = plan.slices == 1 && (plan.kernel == 44 || plan.kernel == 42 || plan.kernel == 22 ||
+                                          plan.kernel == 21 || plan.kernel == 224 || plan.kernel == 214);
+  if (!tiled) {  // the decode-batch kernels and split-K have no fused epilogue: a small tile instead
+    plan = GemmPlan();
+    plan.kernel = M > 64 ? 22 : 21;
+  }
+  return run_gemm(p, plan, fmt, nullptr, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int arcq_scales_from_absmax(float *d_values, int n, float divisor, void *stream) {
+  if (n < 0 || !(divisor > 0.0f)) return ARCQ_ERR_SHAPE;
+  if (n == 0) return ARCQ_OK;
+  if (!d_values) return ARCQ_ERR_NULL;
+  hipLaunchKernelGGL(arcq::scales_from_absmax_kernel, dim3((n + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     d_values, n, divisor);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
 }

@@ -11,6 +11,7 @@
 
 #include "arcq_internal.h"
 #include "arcq_math.h"
+#include "arcq_swiglu.h"
 
 namespace arcq {
 namespace {
@@ -198,14 +199,6 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(QuantParams p) 
 //   pass 2 (reordered)      16 ds_read_u16_d16_hi into registers whose low halves stay zero
 //                           (a bf16 in the high half IS the fp32), amax, scale, encode, 64-bit store
 // ---------------------------------------------------------------------------------------------
-typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
-typedef float v2f __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi) {
-  const v2f v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));  // v_cvt_pk_bf16_f32
-}
-
 // 16 coarse values -> 16 codes with block scale s (r ~ 1/s)
 __device__ __forceinline__ uint2 encode_unit_coarse(const float (&y)[16], float r) {
   float w[16];
@@ -250,14 +243,6 @@ __device__ __forceinline__ float unit_amax3(const float (&v)[16]) {
 template <int FMT>
 __device__ __forceinline__ float scale_rcp(float s) {
   return FMT == ARCQ_FMT_NVFP4 ? __builtin_amdgcn_rcpf(s) : u2f((254u << 23) - f2u(s));
-}
-
-// gamma * h for the two bf16 halves of one register: v_dot2_f32_bf16 with the other half of the
-// gamma operand zeroed gives the exact fp32 product without unpacking h
-__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b) {
-  // the builtin, not a bare inline-asm instruction: the compiler then sees a dot instruction and
-  // keeps the wait states its result needs before another kind of instruction may read it
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, a), __builtin_bit_cast(v2bf, b), 0.0f, false);
 }
 
 // pack_bf16_rne(h_even * gamma_even, h_odd * gamma_odd) for four registers of bf16 pairs.  Written as
@@ -380,28 +365,6 @@ __device__ __forceinline__ void unit_exact(const uint32_t (&yv)[16], float g, ui
     *sb2 = block_scale<FMT>(unit_amax<FMT>(v), &s);
     *pk2 = encode_unit<FMT, false>(v, s);
   }
-}
-
-// act_fn(gate) * up as the reference's layers form it in bf16 (model/qLlamaLayer.py:432,
-// model/qMixtralLayer.py:531): SiLU evaluated in fp32 as x / (1 + exp(-x)) and rounded to bf16,
-// then a bf16 multiply (fp32 product, one rounding).  Two elements per call, packed.
-// The SiLU of a bf16 value has only 65536 possible inputs: the hardware estimates
-// x * rcp(1 + exp2(-x * log2 e)) round to the same bf16 as the library expression for every one of them
-// except 5.9375 and -87.5, -88, -88.5 (all 65536 inputs compared on the GPU; a test repeats it).  Waves
-// that hold one of those, anything of magnitude >= 87, or a NaN take the library expression.
-__device__ __forceinline__ uint32_t silu_pair_bf16(uint32_t gw) {
-  const float g0 = u2f(gw << 16), g1 = u2f(gw & 0xffff0000u);
-  const uint32_t m0 = gw & 0x7fffu, m1 = (gw >> 16) & 0x7fffu;
-  const bool special = m0 >= 0x42aeu || m1 >= 0x42aeu || (gw & 0xffffu) == 0x40beu || (gw >> 16) == 0x40beu;
-  if (__builtin_amdgcn_ballot_w64(special) != 0)
-    return pack_bf16_rne(g0 / (1.0f + expf(-g0)), g1 / (1.0f + expf(-g1)));
-  const float e0 = __builtin_amdgcn_exp2f(g0 * -1.4426950408889634f), e1 = __builtin_amdgcn_exp2f(g1 * -1.4426950408889634f);
-  return pack_bf16_rne(g0 * __builtin_amdgcn_rcpf(1.0f + e0), g1 * __builtin_amdgcn_rcpf(1.0f + e1));
-}
-
-__device__ __forceinline__ uint32_t swiglu_pair(uint32_t gw, uint32_t uw) {
-  const uint32_t a = silu_pair_bf16(gw);
-  return pack_bf16_rne(dot2_bf16(a, uw & 0xffffu), dot2_bf16(a, uw & 0xffff0000u));
 }
 
 template <int FMT, int MODE, bool SCALED, bool GROUPED = false>

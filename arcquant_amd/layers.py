@@ -143,6 +143,16 @@ class QLinearLayer(nn.Module):
             return y.reshape(bsz, q_len, -1)
         return y.reshape(q_len, -1)
 
+    @torch.no_grad()
+    def forward_swiglu(self, x, tensor_scale):
+        """for a gate/up projection whose weight rows alternate gate, up: act_fn(gate) * up [tokens, out/2]
+        straight from the GEMM's epilogue (and its NVFP4 tensor scale when asked), same bits as
+        ``h = self(x); F.silu(h_gate) * h_up``"""
+        qx, scale_x, scale, bsz, q_len = x
+        alpha = (scale, self.scale) if isinstance(scale, torch.Tensor) else (float(scale), self.scale)
+        return agemm.matmul_swiglu(qx, self.W, scale_x, self.scale_w, alpha, fmt=self.quant_type,
+                                   tensor_scale=tensor_scale)
+
 
 class RMSNormQuant(nn.Module):
     """benchmarks/modeling_arc.py:211-227: RMSNorm fused with the activation quantizer; returns the
@@ -197,12 +207,27 @@ def _linear(out_features, in_features, std, device, gen):
 
 class LlamaMLP(nn.Module):
     """SwiGLU MLP with gate and up projections fused into one [2*inter, hidden] linear
-    (model/qLlamaLayer.py:380-443 with the fusion of benchmark configuration 4)."""
+    (model/qLlamaLayer.py:380-443 with the fusion of benchmark configuration 4), followed by the fused
+    SwiGLU -> quantize pass.  interleave=True instead interleaves the fused weight's rows (gate_0, up_0,
+    gate_1, ...) and forms act_fn(gate) * up in the GEMM's epilogue, so that the [tokens, 2*inter] projection
+    output never goes through memory: the same bits, but not the default here, because on one large GEMM with
+    256x256 tiles (one workgroup per CU) the epilogue's activation arithmetic is exposed and costs more than
+    the pass it saves (16384 tokens, MXFP4: 2.01 against 1.73 ms for GEMM + quantizer; NVFP4 3.95 against
+    3.81).  The MoE block's grouped GEMMs run 128x128 tiles, two workgroups per CU, where one workgroup's
+    epilogue hides behind the other's main loop: there it is the default and a gain."""
 
     def __init__(self, gate_up: nn.Linear, down: nn.Linear, select_num_in, select_num_down, in_index, down_index,
-                 quant_type="NVFP4"):
+                 quant_type="NVFP4", interleave=False):
         super().__init__()
         self.inter = down.in_features
+        kp = gate_up.in_features + int(select_num_in)
+        self.interleaved = bool(interleave) and kp % 128 == 0 and kp >= 512 and self.inter % 8 == 0 and \
+            gate_up.bias is None
+        if self.interleaved:
+            w = gate_up.weight.data
+            il = nn.Linear(gate_up.in_features, 2 * self.inter, bias=False, device=w.device, dtype=w.dtype)
+            il.weight.data.copy_(agemm.interleave_gate_up(w[:self.inter], w[self.inter:]))
+            gate_up = il
         self.gate_up_proj = QLinearLayer(gate_up, select_num_in, in_index, quant_type=quant_type)
         self.down_proj = QLinearLayer(down, select_num_down, down_index, quant_type=quant_type)
         self.register_buffer("down_reorder_index", down_index.to(torch.int16))
@@ -211,13 +236,20 @@ class LlamaMLP(nn.Module):
     @torch.no_grad()
     def forward(self, x, residual=None):
         """x: the tuple of the already quantized (normalised) hidden states; residual: added to the output"""
+        sel = self.down_proj.select_num
+        if getattr(self, "interleaved", False):
+            nv = self.quant_type == "NVFP4"
+            r = self.gate_up_proj.forward_swiglu(x, nv)
+            t, scale = r if nv else (r, 1.0)
+            qx, sfx = agemm.reorder_quantize_x(t, self.down_reorder_index, sel, fmt=self.quant_type,
+                                               global_scale=scale if nv else None)
+            return self.down_proj((qx, sfx, scale, x[3], x[4]), residual)
         gu = self.gate_up_proj(x)
         if self.inter <= 16384 and self.inter % 32 == 0:
-            return self.down_proj(swiglu_quantize_tokens(gu, self.inter, self.down_reorder_index,
-                                                         self.down_proj.select_num, self.quant_type), residual)
+            return self.down_proj(swiglu_quantize_tokens(gu, self.inter, self.down_reorder_index, sel, self.quant_type),
+                                  residual)
         t = F.silu(gu[..., :self.inter]) * gu[..., self.inter:]
-        return self.down_proj(quantize_tokens(t, self.down_reorder_index, self.down_proj.select_num, self.quant_type),
-                              residual)
+        return self.down_proj(quantize_tokens(t, self.down_reorder_index, sel, self.quant_type), residual)
 
 
 class LlamaAttention(nn.Module):
@@ -470,13 +502,21 @@ class QLlamaDecoderLayer(nn.Module):
 
 
 class MixtralExpertMLP(nn.Module):
-    """model/qMixtralLayer.py:466-543: w2(act(w1 x) * w3 x) on a ragged set of tokens."""
+    """model/qMixtralLayer.py:466-543: w2(act(w1 x) * w3 x) on a ragged set of tokens.  w1 and w3 share their
+    input and are one quantized linear whose rows alternate w1_0, w3_0, w1_1, ... (act(w1 x) * w3 x then comes
+    out of that GEMM's epilogue); interleave=False stacks them [w1 | w3] with a separate SwiGLU -> quantize pass."""
 
-    def __init__(self, w1: nn.Linear, w3: nn.Linear, w2: nn.Linear, select_num, in_index, w2_index, quant_type="NVFP4"):
+    def __init__(self, w1: nn.Linear, w3: nn.Linear, w2: nn.Linear, select_num, in_index, w2_index, quant_type="NVFP4",
+                 interleave=True):
         super().__init__()
         self.ffn = w1.out_features
+        kp = w1.in_features + int(select_num)
+        self.interleaved = bool(interleave) and kp % 128 == 0 and kp >= 512 and self.ffn % 8 == 0
         w13 = nn.Linear(w1.in_features, 2 * self.ffn, bias=False, device=w1.weight.device, dtype=torch.bfloat16)
-        w13.weight.data.copy_(torch.cat([w1.weight.data, w3.weight.data], dim=0))
+        if self.interleaved:
+            w13.weight.data.copy_(agemm.interleave_gate_up(w1.weight.data, w3.weight.data))
+        else:
+            w13.weight.data.copy_(torch.cat([w1.weight.data, w3.weight.data], dim=0))
         self.w13 = QLinearLayer(w13, select_num, in_index, quant_type=quant_type)   # w1 and w3 share their input
         self.w2 = QLinearLayer(w2, select_num, w2_index, quant_type=quant_type)
         self.register_buffer("w1_reorder_index", in_index.to(torch.int16))
@@ -485,7 +525,15 @@ class MixtralExpertMLP(nn.Module):
 
     @torch.no_grad()
     def forward(self, x):
-        h = self.w13(quantize_tokens(x, self.w1_reorder_index, self.w13.select_num, self.quant_type))
+        xq = quantize_tokens(x, self.w1_reorder_index, self.w13.select_num, self.quant_type)
+        if self.interleaved:
+            nv = self.quant_type == "NVFP4"
+            r = self.w13.forward_swiglu(xq, nv)
+            t, scale = r if nv else (r, 1.0)
+            qx, sfx = agemm.reorder_quantize_x(t, self.w2_reorder_index, self.w2.select_num, fmt=self.quant_type,
+                                               global_scale=scale if nv else None)
+            return self.w2((qx, sfx, scale, None, t.shape[0]))
+        h = self.w13(xq)
         if self.ffn <= 16384 and self.ffn % 32 == 0:
             return self.w2(swiglu_quantize_tokens(h, self.ffn, self.w2_reorder_index, self.w2.select_num,
                                                   self.quant_type))
@@ -512,6 +560,7 @@ class MixtralSparseMoeBlock(nn.Module):
         self.top_k = top_k
         e0 = experts[0]
         same = all(ex.w13.W.shape == e0.w13.W.shape and ex.w2.W.shape == e0.w2.W.shape and
+                   ex.interleaved == e0.interleaved and
                    ex.quant_type == e0.quant_type and ex.w13.select_num == e0.w13.select_num and
                    ex.w2.select_num == e0.w2.select_num and ex.w13.bias is None and ex.w2.bias is None
                    for ex in experts)
@@ -519,7 +568,7 @@ class MixtralSparseMoeBlock(nn.Module):
         self.grouped = bool(grouped) and same and kp13 % 128 == 0 and kp2 % 128 == 0 and min(kp13, kp2) >= 512 and \
             e0.ffn <= 16384 and e0.ffn % 32 == 0 and e0.w13.in_features <= 16384
         if self.grouped:
-            self.quant_type, self.ffn = e0.quant_type, e0.ffn
+            self.quant_type, self.ffn, self.interleaved = e0.quant_type, e0.ffn, e0.interleaved
             for name in ("w13", "w2"):
                 W = torch.stack([getattr(ex, name).W for ex in experts])
                 SF = torch.cat([getattr(ex, name).scale_w for ex in experts])
@@ -547,14 +596,21 @@ class MixtralSparseMoeBlock(nn.Module):
         gs = agemm.grouped_tensor_scale(xs, seg, NVFP4_RANGE) if nv else None
         q, sf = agemm.grouped_reorder_quantize_x(xs, seg, self.w1_reorder_index, e0.w13.select_num, fmt=qt,
                                                  global_scales=gs)
-        h = agemm.grouped_matmul(q, self.w13_W, sf, self.w13_scale_w, seg, gs, self.w13_scale if nv else None, fmt=qt)
-        gate, up = h[:, :self.ffn], h[:, self.ffn:]
-        if nv:
-            q2, sf2, gs2 = agemm.grouped_swiglu_quantize_x(gate, up, seg, self.w2_reorder_index, e0.w2.select_num,
-                                                           fmt=qt, global_scales="absmax")
+        if self.interleaved:          # act(w1 x) * w3 x out of the first GEMM's epilogue, with its per-expert maxima
+            r = agemm.grouped_matmul_swiglu(q, self.w13_W, sf, self.w13_scale_w, seg, gs, self.w13_scale if nv else None,
+                                            fmt=qt, tensor_scale=nv)
+            t, gs2 = r if nv else (r, None)
+            q2, sf2 = agemm.grouped_reorder_quantize_x(t, seg, self.w2_reorder_index, e0.w2.select_num, fmt=qt,
+                                                       global_scales=gs2)
         else:
-            q2, sf2 = agemm.grouped_swiglu_quantize_x(gate, up, seg, self.w2_reorder_index, e0.w2.select_num, fmt=qt)
-            gs2 = None
+            h = agemm.grouped_matmul(q, self.w13_W, sf, self.w13_scale_w, seg, gs, self.w13_scale if nv else None, fmt=qt)
+            gate, up = h[:, :self.ffn], h[:, self.ffn:]
+            if nv:
+                q2, sf2, gs2 = agemm.grouped_swiglu_quantize_x(gate, up, seg, self.w2_reorder_index, e0.w2.select_num,
+                                                               fmt=qt, global_scales="absmax")
+            else:
+                q2, sf2 = agemm.grouped_swiglu_quantize_x(gate, up, seg, self.w2_reorder_index, e0.w2.select_num, fmt=qt)
+                gs2 = None
         return agemm.grouped_matmul(q2, self.w2_W, sf2, self.w2_scale_w, seg, gs2, self.w2_scale if nv else None, fmt=qt)
 
     @torch.no_grad()
@@ -598,7 +654,7 @@ class MixtralSparseMoeBlock(nn.Module):
 
 
 def build_mixtral_block(hidden=4096, ffn=14336, num_experts=8, top_k=2, select_num=128, quant_type="NVFP4",
-                        indices=None, seed=5, device="cuda", grouped=True):
+                        indices=None, seed=5, device="cuda", grouped=True, interleave=True):
     """Random-weight MoE block of benchmark configuration 5; `indices[e]` = (input index, w2 index)."""
     gen = torch.Generator().manual_seed(seed)
     gate = _linear(num_experts, hidden, 1.0 / math.sqrt(hidden), device, gen)
@@ -612,7 +668,7 @@ def build_mixtral_block(hidden=4096, ffn=14336, num_experts=8, top_k=2, select_n
         else:
             i_in = torch.arange(hidden, dtype=torch.int16, device=device)
             i_w2 = torch.arange(ffn, dtype=torch.int16, device=device)
-        experts.append(MixtralExpertMLP(w1, w3, w2, select_num, i_in, i_w2, quant_type))
+        experts.append(MixtralExpertMLP(w1, w3, w2, select_num, i_in, i_w2, quant_type, interleave=interleave))
         del w1, w3, w2
     return MixtralSparseMoeBlock(gate, experts, top_k, grouped=grouped)
 

@@ -238,6 +238,29 @@ int arcq_grouped_matmul(const void *a_codes, const void *a_scales, const void *b
                         const float *d_alpha_a, const float *d_alpha_b, const void *residual, void *c, void *stream);
 
 /*
+ * GEMM with the SwiGLU of the next layer fused into its epilogue, for a fused gate/up projection whose weight
+ * rows ALTERNATE gate_0, up_0, gate_1, up_1, ... (quantize the interleaved bf16 weight with
+ * arcq_reorder_quantize_w): output columns 2j and 2j+1 of a token then sit in one lane, and instead of the
+ * [M, N] projection output the kernel writes t [M, N/2] = act_fn(gate) * up, formed from the bf16-rounded
+ * GEMM outputs exactly as the reference's layers form it from the projection output in bf16
+ * (model/qLlamaLayer.py:432, model/qMixtralLayer.py:531): the same bits as the unfused sequence, without the
+ * projection output passing through memory.  No counterpart in the reference (it names the fusion,
+ * benchmarks/modeling_arc.py:112, and does not ship it).
+ *   d_absmax  NULL, or fp32 [n_seg] ([1] for arcq_matmul_swiglu) zeroed by the caller: receives max |t| per
+ *             expert (as the bits of a non-negative float, i.e. readable as fp32), the numerator of the
+ *             NVFP4 tensor scale of the next quantizer; arcq_scales_from_absmax turns the maxima into
+ *             scales max / divisor in place (1 for a maximum of 0) with an IEEE division
+ *   N multiple of 16; Kp multiple of 128, >= 512; other arguments as for arcq_grouped_matmul / arcq_matmul
+ */
+int arcq_grouped_matmul_swiglu(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,
+                               const int *seg_offsets, int n_seg, int M, int N, int Kp, int fmt, float alpha,
+                               const float *d_alpha_a, const float *d_alpha_b, void *t, float *d_absmax, void *stream);
+int arcq_matmul_swiglu(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
+                       int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b, void *t,
+                       float *d_absmax, void *stream);
+int arcq_scales_from_absmax(float *d_values, int n, float divisor, void *stream);
+
+/*
  * Last step of a mixture-of-experts block: out[t] = sum over token t's experts, in ascending expert number, of
  * bf16(y[row] * weight[row]), every partial sum rounded to bf16 -- what model/qMixtralLayer.py:466-471 gets
  * from `expert(x) * routing_weights[...]` followed by final_hidden_states.index_add_ per expert.  One launch,

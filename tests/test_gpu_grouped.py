@@ -188,3 +188,67 @@ def test_moe_combine_matches_index_add(agemm, top_k):
     position[order] = torch.arange(order.numel())
     got = agemm.moe_combine(y.cuda(), position.cuda(), ws.cuda(), tokens, top_k)
     assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("M,F,K,S", [(300, 256, 512, 128), (64, 384, 448, 64), (1, 128, 512, 0), (2100, 512, 512, 0),
+                                      (700, 1024, 896, 128)])
+def test_matmul_swiglu_equals_unfused_sequence(agemm, fmt, M, F, K, S):
+    """GEMM with the SwiGLU in its epilogue (gate / up weight rows interleaved) against the unfused sequence on
+    the same quantized operands: projection, then silu and multiply in bf16 (torch-ROCm, the pinned reference
+    of tests/test_gpu_swiglu.py); outputs and the tensor scale must be the same bits.  Row counts cover the
+    128x64, 128x128 and 256x256 tiles and ragged last tiles."""
+    import torch.nn.functional as Fn
+    g = torch.Generator().manual_seed(M + F)
+    x = recipes.activations(M, K, seed=9000 + M, outlier_frac=0.01, outlier_gain=40.0).cuda()
+    idx = torch.randperm(K, generator=g).to(torch.int16).cuda()
+    wg = recipes.weights(F, K, seed=9100, std=0.05).cuda()
+    wu = recipes.weights(F, K, seed=9101, std=0.05).cuda()
+    gx = agemm.tensor_scale(x) if fmt == "NVFP4" else None
+    a, sfa = agemm.reorder_quantize_x(x, idx, S, fmt=fmt, global_scale=gx)
+    w_cat = torch.cat([wg, wu])
+    gw = recipes.tensor_scale(w_cat.cpu(), fmt)
+    b_cat, sfb_cat = agemm.reorder_quantize_w(w_cat, idx, S, fmt=fmt, global_scale=gw)
+    b_il, sfb_il = agemm.reorder_quantize_w(agemm.interleave_gate_up(wg, wu), idx, S, fmt=fmt, global_scale=gw)
+    scale = (gx, gw) if fmt == "NVFP4" else 1.0
+    print(f"matmul_swiglu {fmt} M={M} F={F} K={K} S={S}", flush=True)
+    h = agemm.matmul(a, b_cat, sfa, sfb_cat, scale, fmt=fmt)
+    want = Fn.silu(h[:, :F]) * h[:, F:]
+    got, ts = agemm.matmul_swiglu(a, b_il, sfa, sfb_il, scale, fmt=fmt, tensor_scale=True)
+    assert got.shape == (M, F)
+    assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
+    want_ts = want.abs().max().float() / torch.full((), 2688.0, device="cuda")
+    assert float(ts) == float(want_ts if float(want_ts) != 0 else 1.0)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_grouped_matmul_swiglu_equals_unfused_sequence(agemm, fmt):
+    import torch.nn.functional as Fn
+    counts, F, K, S = [5, 0, 170, 1, 300, 0, 64, 9], 256, 512, 128
+    T, E = sum(counts), len(counts)
+    g = torch.Generator().manual_seed(77)
+    x = recipes.activations(T, K, seed=9200, outlier_frac=0.01, outlier_gain=40.0).cuda()
+    seg = segments(counts).cuda()
+    idx = torch.stack([torch.randperm(K, generator=g).to(torch.int16) for _ in range(E)]).cuda()
+    gs = agemm.grouped_tensor_scale(x, seg) if fmt == "NVFP4" else None
+    a, sfa = agemm.grouped_reorder_quantize_x(x, seg, idx, S, fmt=fmt, global_scales=gs)
+    cat, il, gws = [], [], []
+    for e in range(E):
+        wg = recipes.weights(F, K, seed=9300 + e, std=0.05 * (1 + e)).cuda()
+        wu = recipes.weights(F, K, seed=9400 + e, std=0.05).cuda()
+        gw = recipes.tensor_scale(torch.cat([wg, wu]).cpu(), fmt)
+        cat.append(agemm.reorder_quantize_w(torch.cat([wg, wu]), idx[e], S, fmt=fmt, global_scale=gw))
+        il.append(agemm.reorder_quantize_w(agemm.interleave_gate_up(wg, wu), idx[e], S, fmt=fmt, global_scale=gw))
+        gws.append(gw)
+    gw_d = torch.tensor(gws, dtype=torch.float32).cuda() if fmt == "NVFP4" else None
+    stack = lambda pairs: (torch.stack([p[0] for p in pairs]), torch.cat([p[1] for p in pairs]))
+    print(f"grouped matmul_swiglu {fmt}", flush=True)
+    h = agemm.grouped_matmul(a, *stack(cat)[:1], sfa, stack(cat)[1], seg, gs, gw_d, fmt=fmt)
+    want = Fn.silu(h[:, :F]) * h[:, F:]
+    got, ts = agemm.grouped_matmul_swiglu(a, stack(il)[0], sfa, stack(il)[1], seg, gs, gw_d, fmt=fmt, tensor_scale=True)
+    assert torch.equal(got, want)
+    segc = seg.cpu()
+    for e in range(E):
+        rows = want[segc[e]:segc[e + 1]]
+        w = float(rows.abs().max().float() / torch.full((), 2688.0, device="cuda")) if rows.numel() else 0.0
+        assert float(ts[e]) == (w if w != 0.0 else 1.0), e

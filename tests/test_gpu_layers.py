@@ -134,8 +134,32 @@ def test_decoder_layer_matches_fake_quant_flow(layers, fq, fmt):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-@pytest.mark.parametrize("grouped", [True, False])
-def test_mixtral_block_matches_reference_loop(layers, fq, fmt, grouped):
+@pytest.mark.parametrize("tokens", [(2, 24), (1, 1), (3, 100)])
+def test_llama_mlp_fused_swiglu_equals_separate_pass(layers, fmt, tokens):
+    """LlamaMLP with the SwiGLU formed in the gate_up GEMM's epilogue (interleaved weight rows) and with the
+    separate SwiGLU -> quantize pass over [gate | up] (the default): the same bits, residual included"""
+    hidden, inter, S = 384, 768, 128
+    g = torch.Generator().manual_seed(61)
+    gate_up = nn.Linear(hidden, 2 * inter, bias=False, device="cuda", dtype=torch.bfloat16)
+    down = nn.Linear(inter, hidden, bias=False, device="cuda", dtype=torch.bfloat16)
+    gate_up.weight.data.copy_((torch.randn(2 * inter, hidden, generator=g) * 0.05).to(torch.bfloat16))
+    down.weight.data.copy_((torch.randn(hidden, inter, generator=g) * 0.05).to(torch.bfloat16))
+    i_in = torch.randperm(hidden, generator=g).to(torch.int16).cuda()
+    i_down = torch.randperm(inter, generator=g).to(torch.int16).cuda()
+    fused = layers.LlamaMLP(gate_up, down, S, S, i_in, i_down, quant_type=fmt, interleave=True)
+    plain = layers.LlamaMLP(gate_up, down, S, S, i_in, i_down, quant_type=fmt)
+    assert fused.interleaved and not plain.interleaved
+    x = torch.randn(*tokens, hidden, generator=g).to(torch.bfloat16).cuda()
+    res = torch.randn(*tokens, hidden, generator=g).to(torch.bfloat16).cuda()
+    tup = layers.quantize_tokens(x, i_in, S, fmt)
+    print(f"llama mlp fused swiglu {fmt} tokens={tokens}", flush=True)
+    assert torch.equal(fused(tup), plain(tup))
+    assert torch.equal(fused(tup, residual=res), plain(tup, residual=res))
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("grouped,interleave", [(True, True), (True, False), (False, True), (False, False)])
+def test_mixtral_block_matches_reference_loop(layers, fq, fmt, grouped, interleave):
     """The MoE block, as grouped launches over all experts and as the per-expert loop, against the
     reference's loop (model/qMixtralLayer.py:441-471) on the CPU; every expert has its own channel orders."""
     hidden, ffn, E, S = 384, 512, 4, 128
@@ -143,12 +167,13 @@ def test_mixtral_block_matches_reference_loop(layers, fq, fmt, grouped):
     g = torch.Generator().manual_seed(9)
     indices = [(torch.randperm(hidden, generator=g).to(torch.int16).cuda(),
                 torch.randperm(ffn, generator=g).to(torch.int16).cuda()) for _ in range(E)]
-    block = layers.build_mixtral_block(hidden, ffn, E, 2, S, fmt, indices=indices, seed=5, grouped=grouped)
-    assert block.grouped == grouped
+    block = layers.build_mixtral_block(hidden, ffn, E, 2, S, fmt, indices=indices, seed=5, grouped=grouped,
+                                       interleave=interleave)
+    assert block.grouped == grouped and block.experts[0].interleaved == interleave
     x = torch.randn(1, tokens, hidden, generator=g).to(torch.bfloat16)
     logits = torch.randn(tokens, E, generator=g)
     logits[:, 3] -= 100.0                                   # an expert that receives no token
-    print(f"mixtral block {fmt} grouped={grouped}", flush=True)
+    print(f"mixtral block {fmt} grouped={grouped} interleave={interleave}", flush=True)
     y, _ = block(x.cuda(), router_logits=logits.cuda())
     assert y.shape == x.shape
 
@@ -166,6 +191,8 @@ def test_mixtral_block_matches_reference_loop(layers, fq, fmt, grouped):
         ex = block.experts[e]
         ih, ii = indices[e][0].cpu(), indices[e][1].cpu()
         w13 = (agemm.dequantize(ex.w13.W.contiguous(), ex.w13.scale_w.contiguous(), fmt=fmt) * ex.w13.scale).cpu()
+        if ex.interleaved:                                  # rows w1_0, w3_0, w1_1, ... -> [w1 | w3]
+            w13 = torch.cat([w13[0::2], w13[1::2]])
         w2 = (agemm.dequantize(ex.w2.W.contiguous(), ex.w2.scale_w.contiguous(), fmt=fmt) * ex.w2.scale).cpu()
         cur = x2[top_x]
         hcur = (ref_quant_x(fq, cur, ih, S, fmt) @ w13.T).to(torch.bfloat16)
