@@ -311,19 +311,20 @@ __device__ __forceinline__ void wait_dma_and_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-template <int WN, int WM>
+template <int WN, int WM, int NWM>
 __device__ __forceinline__ void store_workgroup_tile_swiglu_fwd(const GemmParams &p, v16f (&acc)[WN][WM], uint8_t *ldsA,
                                                                 uint8_t *ldsB, int m_base, int n_base, int wave, int lane);
 
 // Epilogue shared by the tiled kernels: acc[i][j] is the 32x32 tile (n-tile i, m-tile j) of the
-// wave tile.  ldsA / ldsB: two LDS areas of at least 2*32*WM*64*WN bytes each, free for reuse.
-template <int WN, int WM>
+// wave tile.  The workgroup's waves form a 2 (along N) x NWM (along M) grid, wave = n + 2 * m.
+// ldsA / ldsB: two LDS areas of at least NWM*32*WM*64*WN bytes each, free for reuse.
+template <int WN, int WM, int NWM = 2>
 __device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (&acc)[WN][WM], uint8_t *ldsA,
                                                      uint8_t *ldsB, int m_base, int n_base, int wave, int lane) {
-  constexpr int BN = 64 * WN, BM = 64 * WM;
+  constexpr int BN = 64 * WN, BM = 32 * WM * NWM;
   const int r = lane & 31, kh = lane >> 5;
   const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;
-  if (p.swiglu) return store_workgroup_tile_swiglu_fwd<WN, WM>(p, acc, ldsA, ldsB, m_base, n_base, wave, lane);
+  if (p.swiglu) return store_workgroup_tile_swiglu_fwd<WN, WM, NWM>(p, acc, ldsA, ldsB, m_base, n_base, wave, lane);
   if (p.partial) {  // split-K: the unscaled fp32 tile of this K range
     float *part = p.partial + (size_t)blockIdx.y * p.M * p.N;
 #pragma unroll
@@ -356,7 +357,7 @@ __device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (
     wait_dma_and_sync();  // every wave is done reading operands
     constexpr int RB = 64 * WN;                       // bytes per row of the wave tile
     constexpr int LPR = 4 * WN;                       // lanes per row when reading 16 bytes each
-    uint8_t *region = (wave < 2 ? ldsA : ldsB) + (wave & 1) * (32 * WM * RB);
+    uint8_t *region = (wave < NWM ? ldsA : ldsB) + (wave % NWM) * (32 * WM * RB);
 #pragma unroll
     for (int i = 0; i < WN; ++i)
 #pragma unroll
@@ -400,10 +401,10 @@ __device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (
 // (gate_j, up_j, gate_j+1, up_j+1); each is rounded to bf16 as the plain epilogue would store it, and the two
 // products act_fn(gate) * up leave as one dword.  Whole tiles go through LDS so that every store
 // instruction writes 16 bytes per lane along output rows; ragged tiles store dwords with bounds checks.
-template <int WN, int WM>
+template <int WN, int WM, int NWM>
 __device__ __forceinline__ void store_workgroup_tile_swiglu(const GemmParams &p, v16f (&acc)[WN][WM], uint8_t *ldsA,
                                                             uint8_t *ldsB, int m_base, int n_base, int wave, int lane) {
-  constexpr int BN = 64 * WN, BM = 64 * WM;
+  constexpr int BN = 64 * WN, BM = 32 * WM * NWM;
   const int r = lane & 31, kh = lane >> 5;
   const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;
   const float alpha = effective_alpha(p);
@@ -423,7 +424,7 @@ __device__ __forceinline__ void store_workgroup_tile_swiglu(const GemmParams &p,
     wait_dma_and_sync();  // every wave is done reading operands
     constexpr int RB = 32 * WN;   // bytes per row of the wave tile: 16 * WN products
     constexpr int LPR = 2 * WN;   // lanes per row when reading 16 bytes each
-    uint8_t *region = (wave < 2 ? ldsA : ldsB) + (wave & 1) * (32 * WM * RB);
+    uint8_t *region = (wave < NWM ? ldsA : ldsB) + (wave % NWM) * (32 * WM * RB);
 #pragma unroll
     for (int i = 0; i < WN; ++i)
 #pragma unroll
@@ -474,10 +475,10 @@ __device__ __forceinline__ void store_workgroup_tile_swiglu(const GemmParams &p,
   }
 }
 
-template <int WN, int WM>
+template <int WN, int WM, int NWM>
 __device__ __forceinline__ void store_workgroup_tile_swiglu_fwd(const GemmParams &p, v16f (&acc)[WN][WM], uint8_t *ldsA,
                                                                 uint8_t *ldsB, int m_base, int n_base, int wave, int lane) {
-  store_workgroup_tile_swiglu<WN, WM>(p, acc, ldsA, ldsB, m_base, n_base, wave, lane);
+  store_workgroup_tile_swiglu<WN, WM, NWM>(p, acc, ldsA, ldsB, m_base, n_base, wave, lane);
 }
 
 // An FP4 operand of the scaled MFMA is 4 registers; the builtin's type has 8, the upper 4 unused.
@@ -486,10 +487,12 @@ __device__ __forceinline__ v8i fp4_operand(uint4 q) {
   return __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1);
 }
 
-template <int WN, int WM, int NS = 2>
-__global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
-  constexpr int BN = 64 * WN, BM = 64 * WM;
-  static_assert(NS == 2 || (NS == 4 && WN == 2 && WM <= 2), "the four-stage ring's wait counts are those of the 128x64 and 128x128 tiles");
+template <int WN, int WM, int NS = 2, int NWM = 2>
+__global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
+  // waves: 2 along N x NWM along M (wave = n + 2 * m), each with WN x WM accumulator tiles of 32 x 32
+  constexpr int BN = 64 * WN, BM = 32 * WM * NWM, NW = 2 * NWM;
+  constexpr int RPI = 16 * NWM;  // rows of 128 code bytes that one load instruction of the workgroup covers
+  static_assert(NS == 2 || (NS == 4 && WN == 2 && WM <= 2 && NWM == 2), "the four-stage ring's wait counts are those of the 128x64 and 128x128 tiles");
   __shared__ uint4 sW[NS * BN * 8], sX[NS * BM * 8];  // code tiles, NS stages each
   __shared__ uint4 sWs[NS * BN], sXs[NS * BM];        // 16 scale bytes per row (two K steps), NS stages each
   const int tid = threadIdx.x, lane = tid & 63;
@@ -514,26 +517,26 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
   const bool short_last = (p.Kp & 255) != 0;  // then the last step has 4 valid blocks (K' % 256 == 128)
 
   // ---- global -> LDS plan: codes
-  const int ld_row = tid >> 3;                                   // + 32*i
+  const int ld_row = tid >> 3;                                   // + RPI*i
   const int ld_q = (tid & 7) ^ ((ld_row >> 1) & 7);              // chunk fetched by this lane
-  const uint8_t *wsrc[WN * 2], *xsrc[WM * 2];
+  const uint8_t *wsrc[BN / RPI], *xsrc[BM / RPI];
 #pragma unroll
-  for (int i = 0; i < WN * 2; ++i)
-    wsrc[i] = p.b_codes + (size_t)min(n_base + 32 * i + ld_row, p.N - 1) * kbytes + ld_q * 16;
+  for (int i = 0; i < BN / RPI; ++i)
+    wsrc[i] = p.b_codes + (size_t)min(n_base + RPI * i + ld_row, p.N - 1) * kbytes + ld_q * 16;
 #pragma unroll
-  for (int i = 0; i < WM * 2; ++i)
-    xsrc[i] = p.a_codes + (size_t)min(m_base + 32 * i + ld_row, p.M - 1) * kbytes + ld_q * 16;
+  for (int i = 0; i < BM / RPI; ++i)
+    xsrc[i] = p.a_codes + (size_t)min(m_base + RPI * i + ld_row, p.M - 1) * kbytes + ld_q * 16;
   // ---- scales: a lane fetches 16 bytes = the E8M0 bytes of one row for a PAIR of K steps; one
   // load instruction covers 64 rows.  Instruction j of the weights goes to wave j%4, of the
   // activations to wave (j+WN)%4.  If the row ends inside the last pair, the 16-byte window is
   // shifted back to end at the row end (sc_shift bytes; K' % 128 == 0 makes it a multiple of 4).
   const int npairs = (nk + 1) >> 1;
   const int sc_shift = max(0, npairs * 16 - ksc);
-  const uint8_t *wssrc[WN], *xssrc[WM];
+  const uint8_t *wssrc[BN / 64], *xssrc[BM / 64];
 #pragma unroll
-  for (int j = 0; j < WN; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
+  for (int j = 0; j < BN / 64; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
 #pragma unroll
-  for (int j = 0; j < WM; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
+  for (int j = 0; j < BM / 64; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
   const uint32_t lw0 = (uint32_t)reinterpret_cast<uintptr_t>(sW) + wave * 1024;
   const uint32_t lx0 = (uint32_t)reinterpret_cast<uintptr_t>(sX) + wave * 1024;
   const uint32_t lws0 = (uint32_t)reinterpret_cast<uintptr_t>(sWs);
@@ -546,18 +549,18 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
     const bool clip = short_last && kt == nk - 1;
     const int koff = kt * 128 - ((clip && ld_q >= 4) ? 64 : 0);
 #pragma unroll
-    for (int i = 0; i < WN * 2; ++i) lds_dma16(wsrc[i] + koff, lw0 + st * (BN * 128) + i * 4096);
+    for (int i = 0; i < BN / RPI; ++i) lds_dma16(wsrc[i] + koff, lw0 + st * (BN * 128) + i * (RPI * 128));
 #pragma unroll
-    for (int i = 0; i < WM * 2; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * 4096);
+    for (int i = 0; i < BM / RPI; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * (RPI * 128));
     if ((kt & 1) == 0) {  // scales of steps kt and kt+1
       const int pair = kt >> 1, sst = pair & (NS - 1);
       const int soff = pair * 16 - (pair == npairs - 1 ? sc_shift : 0);
 #pragma unroll
-      for (int j = 0; j < WN; ++j)
-        if ((j & 3) == wave) lds_dma16(wssrc[j] + soff, lws0 + sst * (BN * 16) + j * 1024);
+      for (int j = 0; j < BN / 64; ++j)
+        if ((j % NW) == wave) lds_dma16(wssrc[j] + soff, lws0 + sst * (BN * 16) + j * 1024);
 #pragma unroll
-      for (int j = 0; j < WM; ++j)
-        if (((j + WN) & 3) == wave) lds_dma16(xssrc[j] + soff, lxs0 + sst * (BM * 16) + j * 1024);
+      for (int j = 0; j < BM / 64; ++j)
+        if (((j + BN / 64) % NW) == wave) lds_dma16(xssrc[j] + soff, lxs0 + sst * (BM * 16) + j * 1024);
     }
   };
 
@@ -673,8 +676,8 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_tiled(GemmParams p) {
     compute(nk - 1, std::true_type{});
   }
 
-  store_workgroup_tile<WN, WM>(p, acc, reinterpret_cast<uint8_t *>(sW), reinterpret_cast<uint8_t *>(sX), m_base, n_base,
-                               wave, lane);
+  store_workgroup_tile<WN, WM, NWM>(p, acc, reinterpret_cast<uint8_t *>(sW), reinterpret_cast<uint8_t *>(sX), m_base,
+                                    n_base, wave, lane);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -721,9 +724,11 @@ __device__ __forceinline__ v8h decode8_nvfp4_f16(uint32_t codes, uint32_t scale_
   return __builtin_bit_cast(v8h, d);
 }
 
-template <int WN, int WM>
-__global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
-  constexpr int BN = 64 * WN, BM = 64 * WM;
+template <int WN, int WM, int NWM = 2>
+__global__ __launch_bounds__(128 * NWM) void gemm_nvfp4_tiled(GemmParams p) {
+  // waves: 2 along N x NWM along M (wave = n + 2 * m), each with WN x WM accumulator tiles of 32 x 32
+  constexpr int BN = 64 * WN, BM = 32 * WM * NWM, NW = 2 * NWM;
+  constexpr int RPI = 16 * NWM;  // rows of 128 code bytes that one load instruction of the workgroup covers
   __shared__ uint4 sW[2 * BN * 8], sX[2 * BM * 8];  // code tiles, two stages each
   __shared__ uint4 sWs[2 * BN], sXs[2 * BM];        // 16 scale bytes per row per K step, two stages each
   const int tid = threadIdx.x, lane = tid & 63;
@@ -747,21 +752,21 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
 
   const int ld_row = tid >> 3;
   const int ld_q = (tid & 7) ^ ((ld_row >> 1) & 7);
-  const uint8_t *wsrc[WN * 2], *xsrc[WM * 2];
+  const uint8_t *wsrc[BN / RPI], *xsrc[BM / RPI];
 #pragma unroll
-  for (int i = 0; i < WN * 2; ++i)
-    wsrc[i] = p.b_codes + (size_t)min(n_base + 32 * i + ld_row, p.N - 1) * kbytes + ld_q * 16;
+  for (int i = 0; i < BN / RPI; ++i)
+    wsrc[i] = p.b_codes + (size_t)min(n_base + RPI * i + ld_row, p.N - 1) * kbytes + ld_q * 16;
 #pragma unroll
-  for (int i = 0; i < WM * 2; ++i)
-    xsrc[i] = p.a_codes + (size_t)min(m_base + 32 * i + ld_row, p.M - 1) * kbytes + ld_q * 16;
+  for (int i = 0; i < BM / RPI; ++i)
+    xsrc[i] = p.a_codes + (size_t)min(m_base + RPI * i + ld_row, p.M - 1) * kbytes + ld_q * 16;
   // scales: one lane = the 16 scale bytes of one row for this K step; instruction j (64 rows) of
   // the weights goes to wave j%4, of the activations to wave (j+WN)%4.  In a short last step the
   // window is shifted back by 8 bytes so that it ends with the row.
-  const uint8_t *wssrc[WN], *xssrc[WM];
+  const uint8_t *wssrc[BN / 64], *xssrc[BM / 64];
 #pragma unroll
-  for (int j = 0; j < WN; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
+  for (int j = 0; j < BN / 64; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
 #pragma unroll
-  for (int j = 0; j < WM; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
+  for (int j = 0; j < BM / 64; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
   const uint32_t lw0 = (uint32_t)reinterpret_cast<uintptr_t>(sW) + wave * 1024;
   const uint32_t lx0 = (uint32_t)reinterpret_cast<uintptr_t>(sX) + wave * 1024;
   const uint32_t lws0 = (uint32_t)reinterpret_cast<uintptr_t>(sWs);
@@ -773,15 +778,15 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
     const int koff = kt * 128 - ((clip && ld_q >= 4) ? 64 : 0);
     const int soff = kt * 16 - (clip ? 8 : 0);
 #pragma unroll
-    for (int i = 0; i < WN * 2; ++i) lds_dma16(wsrc[i] + koff, lw0 + st * (BN * 128) + i * 4096);
+    for (int i = 0; i < BN / RPI; ++i) lds_dma16(wsrc[i] + koff, lw0 + st * (BN * 128) + i * (RPI * 128));
 #pragma unroll
-    for (int i = 0; i < WM * 2; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * 4096);
+    for (int i = 0; i < BM / RPI; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * (RPI * 128));
 #pragma unroll
-    for (int j = 0; j < WN; ++j)
-      if ((j & 3) == wave) lds_dma16(wssrc[j] + soff, lws0 + st * (BN * 16) + j * 1024);
+    for (int j = 0; j < BN / 64; ++j)
+      if ((j % NW) == wave) lds_dma16(wssrc[j] + soff, lws0 + st * (BN * 16) + j * 1024);
 #pragma unroll
-    for (int j = 0; j < WM; ++j)
-      if (((j + WN) & 3) == wave) lds_dma16(xssrc[j] + soff, lxs0 + st * (BM * 16) + j * 1024);
+    for (int j = 0; j < BM / 64; ++j)
+      if (((j + BN / 64) % NW) == wave) lds_dma16(xssrc[j] + soff, lxs0 + st * (BM * 16) + j * 1024);
   };
 
   const int r = lane & 31, kh = lane >> 5;
@@ -901,8 +906,8 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_tiled(GemmParams p) {
     wait_dma_and_sync();
     compute(nk - 1, std::true_type{});
   }
-  store_workgroup_tile<WN, WM>(p, acc, reinterpret_cast<uint8_t *>(sW), reinterpret_cast<uint8_t *>(sX), m_base, n_base,
-                               wave, lane);
+  store_workgroup_tile<WN, WM, NWM>(p, acc, reinterpret_cast<uint8_t *>(sW), reinterpret_cast<uint8_t *>(sX), m_base,
+                                    n_base, wave, lane);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1106,24 +1111,24 @@ int launch_skinny_for(const GemmParams &p, hipStream_t st) {
   return launch_skinny<FMT, 4, 1>(p, st);
 }
 
-template <int WN, int WM>
+template <int WN, int WM, int NWM = 2>
 int launch_nvfp4_tiled(const GemmParams &p, hipStream_t st) {
-  constexpr int BN = 64 * WN, BM = 64 * WM;
+  constexpr int BN = 64 * WN, BM = 32 * WM * NWM;
   // grouped: every segment may end in one partial tile of rows
   const int total = ((p.M + BM - 1) / BM + (p.seg ? p.n_seg : 0)) * ((p.N + BN - 1) / BN);
   const int grid = ((total + 7) / 8) * 8;
-  hipLaunchKernelGGL((gemm_nvfp4_tiled<WN, WM>), dim3(grid, p.k_slices), dim3(256), 0, st, p);
+  hipLaunchKernelGGL((gemm_nvfp4_tiled<WN, WM, NWM>), dim3(grid, p.k_slices), dim3(128 * NWM), 0, st, p);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }
 
-template <int WN, int WM, int NS = 2>
+template <int WN, int WM, int NS = 2, int NWM = 2>
 int launch_mxfp4_tiled(const GemmParams &p, hipStream_t st) {
-  constexpr int BN = 64 * WN, BM = 64 * WM;
+  constexpr int BN = 64 * WN, BM = 32 * WM * NWM;
   // grouped: every segment may end in one partial tile of rows
   const int total = ((p.M + BM - 1) / BM + (p.seg ? p.n_seg : 0)) * ((p.N + BN - 1) / BN);
   const int grid = ((total + 7) / 8) * 8;  // whole groups of 8 so that the XCD split covers every tile
-  hipLaunchKernelGGL((gemm_mxfp4_tiled<WN, WM, NS>), dim3(grid, p.k_slices), dim3(256), 0, st, p);
+  hipLaunchKernelGGL((gemm_mxfp4_tiled<WN, WM, NS, NWM>), dim3(grid, p.k_slices), dim3(128 * NWM), 0, st, p);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }
@@ -1214,11 +1219,13 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
   const bool tiled_ok = fast_ok && Kp >= 512;
   if (fmt == ARCQ_FMT_MXFP4 && force != 0 && tiled_ok) {
     // Tile choice from a small cost model: rounds of resident workgroups x cost of one round.
-    // 256x256 tiles run ~1.3x faster per flop than 256x128 ones (LDS reads per MFMA) and 128x128
-    // ones ~0.75x; 128x128 workgroups fit two to a CU.  Units: a 256x128 tile = 2.
+    // 256x256 tiles run ~1.4x faster per flop than 256x128 ones (LDS reads per MFMA) and 128x128
+    // ones ~0.75x; 128x128 workgroups fit two to a CU.  Units: a 256x128 tile = 2.  The 256x256 tile runs as
+    // eight waves of 128x64 (kernel 84; two waves per SIMD: one wave's waits for LDS data and for the next
+    // stage overlap with the other's MFMAs), 7-16 % faster than as four waves of 128x128 (kernel 44).
     const long t44 = (long)((M + 255) / 256) * ((N + 255) / 256), t42 = (long)((M + 127) / 128) * ((N + 255) / 256);
     const long t22 = (long)((M + 127) / 128) * ((N + 127) / 128);
-    const double c44 = (double)((t44 + 255) / 256) * 3.08, c42 = (double)((t42 + 255) / 256) * 2.0;
+    const double c44 = (double)((t44 + 255) / 256) * 2.8, c42 = (double)((t42 + 255) / 256) * 2.0;
     const double c22 = t22 <= 256 ? 1.33 : (double)((t22 + 511) / 512) * 2.67;
     // Problems of one round of workgroups are bounded by the memory latency of their K steps, not by
     // the matrix cores: the smallest tile that still fits one round (most CUs busy), with three K steps
@@ -1229,7 +1236,7 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
                                 : (t22 <= 256 ? 224
                                               : (M <= 128 ? 21
                                                           : (M < 512 ? 22
-                                                                     : (c44 < c42 && c44 < c22 ? 44 : (c42 <= c22 ? 42 : 22)))));
+                                                                     : (c44 < c42 && c44 < c22 ? 84 : (c42 <= c22 ? 42 : 22)))));
     plan.kernel = force > 1 ? force : pick;
     return plan;
   }
@@ -1263,6 +1270,7 @@ int run_gemm(GemmParams p, const GemmPlan &plan, int fmt, float *scratch, hipStr
   if (fmt == ARCQ_FMT_MXFP4) {
     switch (plan.kernel) {
       case 44: return launch_mxfp4_tiled<4, 4>(p, st);
+      case 84: return launch_mxfp4_tiled<4, 2, 2, 4>(p, st);  // 256x256 tile, eight waves of 128x64
       case 42: return launch_mxfp4_tiled<4, 2>(p, st);
       case 224: return launch_mxfp4_tiled<2, 2, 4>(p, st);
       case 22: return launch_mxfp4_tiled<2, 2>(p, st);
@@ -1273,6 +1281,7 @@ int run_gemm(GemmParams p, const GemmPlan &plan, int fmt, float *scratch, hipStr
   } else {
     switch (plan.kernel) {
       case 44: return launch_nvfp4_tiled<4, 4>(p, st);
+      case 84: return launch_nvfp4_tiled<4, 2, 4>(p, st);  // 256x256 tile, eight waves of 128x64
       case 42: return launch_nvfp4_tiled<4, 2>(p, st);
       case 22: return launch_nvfp4_tiled<2, 2>(p, st);
       case 21: return launch_nvfp4_tiled<2, 1>(p, st);
@@ -1450,8 +1459,8 @@ int grouped_matmul_impl(const void *a_codes, const void *a_scales, const void *b
   const int avg = M / n_seg;
   GemmPlan plan;
   const int force = tuning().gemm_kernel;
-  plan.kernel = avg >= 2048 ? 44 : (avg >= 96 ? 22 : 21);
-  if (force == 44 || force == 42 || force == 22 || force == 21) plan.kernel = force;
+  plan.kernel = avg >= 2048 ? (fmt == ARCQ_FMT_MXFP4 ? 84 : 44) : (avg >= 96 ? 22 : 21);
+  if (force == 84 || force == 44 || force == 42 || force == 22 || force == 21) plan.kernel = force;
   return run_gemm(p, plan, fmt, nullptr, static_cast<hipStream_t>(stream));
 }
 
@@ -1494,7 +1503,7 @@ extern "C" int arcq_matmul_swiglu(const void *a_codes, const void *a_scales, con
   p.swiglu = 1;
   p.absmax_bits = reinterpret_cast<uint32_t *>(d_absmax);
   GemmPlan plan = plan_gemm(M, N, Kp, fmt, true);
-  const bool tiled = plan.slices == 1 && (plan.kernel == 44 || plan.kernel == 42 || plan.kernel == 22 ||
+  const bool tiled = plan.slices == 1 && (plan.kernel == 84 || plan.kernel == 44 || plan.kernel == 42 || plan.kernel == 22 ||
                                           plan.kernel == 21 || plan.kernel == 224 || plan.kernel == 214);
   if (!tiled) {  // the decode-batch kernels and split-K have no fused epilogue: a small tile instead
     plan = GemmPlan();
