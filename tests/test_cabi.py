@@ -64,3 +64,43 @@ def test_null_alignment_and_matmul_errors():
     assert L.arcq_matmul(ok, None, ok, ok, 4, 4, 128, 0, 1.0, None, None, ok, None) == 1
     assert L.arcq_matmul(ok, ok, ok, ok, 0, 4, 128, 0, 1.0, None, None, ok, None) == 0
     assert b"16-byte" in L.arcq_status_string(4)
+
+
+def test_grouped_entry_points_reject_bad_arguments():
+    """the MoE entry points check shapes, pointers and alignment before any launch"""
+    L = _lib.lib()
+    ok, odd = ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1004)
+    gq = L.arcq_grouped_reorder_quantize_x
+    assert gq(ok, 8, 4096, ok, 0, ok, 128, 0, None, ok, ok, None) == 2          # no segment
+    assert gq(ok, 8, 4100, ok, 2, ok, 128, 0, None, ok, ok, None) == 2          # K % 32
+    assert gq(ok, 8, 4096, ok, 2, ok, 8, 0, None, ok, ok, None) == 2            # select_num % 16
+    assert gq(ok, 8, 4096, ok, 2, ok, 128, 7, None, ok, ok, None) == 3          # format
+    assert gq(ok, 8, 4096, None, 2, ok, 128, 0, None, ok, ok, None) == 1        # no offsets
+    assert gq(odd, 8, 4096, ok, 2, ok, 128, 0, None, ok, ok, None) == 4
+    assert gq(ok, 0, 4096, ok, 2, ok, 128, 0, None, ok, ok, None) == 0          # no rows: nothing to do
+    gs = L.arcq_grouped_swiglu_quantize_x
+    assert gs(ok, ok, 4000, 8, 4096, ok, 2, ok, 128, 0, None, ok, ok, None) == 2  # row stride below K
+    assert gs(ok, None, 8192, 8, 4096, ok, 2, ok, 128, 0, None, ok, ok, None) == 1
+    ts = L.arcq_grouped_tensor_scale
+    assert ts(ok, None, 4096, 8, 4096, ok, 0, 2688.0, ok, None) == 2
+    assert ts(ok, None, 4096, 8, 4096, ok, 2, 0.0, ok, None) == 2
+    assert ts(ok, None, 4096, 8, 4096, ok, 2, 2688.0, None, None) == 1
+    gm = L.arcq_grouped_matmul
+    assert gm(ok, ok, ok, ok, ok, 2, 8, 256, 448, 1, 1.0, None, None, None, ok, None) == 2    # K' % 128
+    assert gm(ok, ok, ok, ok, ok, 2, 8, 256, 384, 1, 1.0, None, None, None, ok, None) == 2    # K' < 512
+    assert gm(ok, ok, ok, ok, ok, 0, 8, 256, 512, 1, 1.0, None, None, None, ok, None) == 2    # no segment
+    assert gm(ok, ok, ok, ok, None, 2, 8, 256, 512, 1, 1.0, None, None, None, ok, None) == 1
+    assert gm(ok, odd, ok, ok, ok, 2, 8, 256, 512, 1, 1.0, None, None, None, ok, None) == 4   # scale bytes unaligned
+    assert gm(ok, ok, ok, ok, ok, 2, 0, 256, 512, 1, 1.0, None, None, None, ok, None) == 0
+    sw = L.arcq_grouped_matmul_swiglu
+    assert sw(ok, ok, ok, ok, ok, 2, 8, 250, 512, 1, 1.0, None, None, ok, None, None) == 2    # N % 16
+    assert L.arcq_matmul_swiglu(ok, ok, ok, ok, 8, 256, 448, 1, 1.0, None, None, ok, None, None) == 2
+    assert L.arcq_scales_from_absmax(None, 4, 2688.0, None) == 1
+    assert L.arcq_scales_from_absmax(ok, 4, -1.0, None) == 2
+    mc = L.arcq_moe_combine
+    assert mc(ok, ok, ok, 8, 4100, 2, 16, ok, None) == 2                                      # H % 8
+    assert mc(ok, ok, ok, 8, 4096, 9, 72, ok, None) == 2                                      # top_k > 8
+    assert mc(ok, None, ok, 8, 4096, 2, 16, ok, None) == 1
+    assert mc(ok, ok, ok, 0, 4096, 2, 0, ok, None) == 0
+    assert L.arcq_stream_probe_variants() >= 2
+    assert L.arcq_stream_probe_variant(ok, ok, 1024, 512, 99, None) == 2
