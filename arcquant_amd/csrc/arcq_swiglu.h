@@ -43,6 +43,12 @@ __device__ __forceinline__ uint32_t silu_pair_bf16(uint32_t gw) {
 
 __device__ __forceinline__ uint32_t swiglu_pair(uint32_t gw, uint32_t uw) {
   const uint32_t a = silu_pair_bf16(gw);
+  // The dot instruction adds (other half) * 0 to each product: an infinite or NaN activation in one half would
+  // turn its neighbour's product into NaN where torch's elementwise multiply leaves it alone.  Waves that hold
+  // one (a vote, as for the special values above) multiply the unpacked halves instead: the same bits otherwise.
+  const bool nonfinite = (a & 0x7f80u) == 0x7f80u || (a & 0x7f800000u) == 0x7f800000u;
+  if (__builtin_amdgcn_ballot_w64(nonfinite) != 0)
+    return pack_bf16_rne(u2f(a << 16) * u2f(uw << 16), u2f(a & 0xffff0000u) * u2f(uw & 0xffff0000u));
   return pack_bf16_rne(dot2_bf16(a, uw & 0xffffu), dot2_bf16(a, uw & 0xffff0000u));
 }
 

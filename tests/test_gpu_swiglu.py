@@ -65,6 +65,33 @@ def test_fused_equals_unfused_on_gpu(agemm, oracle, fmt, M, K, S):
     assert dc <= 1e-3 and ds <= 1e-3, (dc, ds)
 
 
+def test_infinite_gate_leaves_its_neighbour_alone(agemm):
+    """The kernels form the products of a pair of elements with a dot instruction whose unused term is
+    (other half) * 0: an infinite activation would turn its neighbour's product into NaN there.  Waves that
+    hold a non-finite activation multiply the unpacked halves instead, as torch's elementwise silu * up does:
+    max |t| of an eight-element row around such a pair is the infinity itself, not NaN."""
+    import ctypes
+    from arcquant_amd import _lib
+    L = _lib.lib()
+    inf = float("inf")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for gate in ([inf, 2.0, 1, 1, 1, 1, 1, 1], [2.0, inf, 1, 1, 1, 1, 1, 1], [1, 1, 1, 1, 1, 1, 3.0, inf]):
+        g = torch.tensor(gate, dtype=torch.bfloat16, device="cuda")
+        u = torch.full((8,), 0.5, dtype=torch.bfloat16, device="cuda")
+        want = (F.silu(g) * u).abs().float()
+        assert int(torch.isinf(want).sum()) == 1 and not bool(torch.isnan(want).any())     # torch: one inf, no NaN
+        out = torch.zeros((), dtype=torch.float32, device="cuda")
+        assert L.arcq_tensor_scale(g.data_ptr(), u.data_ptr(), 8, 1, 8, 1.0, out.data_ptr(), stream) == 0
+        torch.cuda.synchronize()
+        assert float(out) == inf, (gate, float(out))          # a NaN neighbour would win the maximum (its bits are larger)
+    # and the finite neighbour's value is what it is without the infinity beside it
+    g = torch.tensor([0.0, 2.0, 0, 0, 0, 0, 0, 0], dtype=torch.bfloat16, device="cuda")
+    u = torch.full((8,), 0.5, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros((), dtype=torch.float32, device="cuda")
+    assert L.arcq_tensor_scale(g.data_ptr(), u.data_ptr(), 8, 1, 8, 1.0, out.data_ptr(), stream) == 0
+    assert float(out) == float((F.silu(g) * u).abs().max())
+
+
 def test_errors(agemm):
     g = torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda")
     idx = torch.arange(64, dtype=torch.int16, device="cuda")
@@ -79,8 +106,7 @@ def test_errors(agemm):
 def test_silu_of_every_bf16_value(agemm):
     """The SiLU inside the fused kernels against torch's own bf16 silu on the GPU for all 65536 bf16
     inputs: arcq_tensor_scale over a tensor of eight copies of g with up = 1 and divisor 1 returns
-    |silu(g)| itself.  Finite inputs only: the kernels form the product with `up` through a two-term dot
-    product whose unused term is x * 0, which turns an infinite x into NaN."""
+    |silu(g)| itself.  Finite inputs here; test_infinite_gate_leaves_its_neighbour_alone covers the others."""
     import ctypes
     from arcquant_amd import _lib
     L = _lib.lib()
