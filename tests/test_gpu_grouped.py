@@ -192,12 +192,12 @@ def test_moe_combine_matches_index_add(agemm, top_k):
 
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("M,F,K,S", [(300, 256, 512, 128), (64, 384, 448, 64), (1, 128, 512, 0), (2100, 512, 512, 0),
-                                      (700, 1024, 896, 128)])
+                                      (700, 1024, 896, 128), (2100, 2048, 512, 0), (4000, 1024, 512, 0)])
 def test_matmul_swiglu_equals_unfused_sequence(agemm, fmt, M, F, K, S):
     """GEMM with the SwiGLU in its epilogue (gate / up weight rows interleaved) against the unfused sequence on
     the same quantized operands: projection, then silu and multiply in bf16 (torch-ROCm, the pinned reference
     of tests/test_gpu_swiglu.py); outputs and the tensor scale must be the same bits.  Row counts cover the
-    128x64, 128x128 and 256x256 tiles and ragged last tiles."""
+    128x64, 128x128, 256x128 and 256x256 tiles (the last two as eight waves for MXFP4) and ragged last tiles."""
     import torch.nn.functional as Fn
     g = torch.Generator().manual_seed(M + F)
     x = recipes.activations(M, K, seed=9000 + M, outlier_frac=0.01, outlier_gain=40.0).cuda()
@@ -222,9 +222,10 @@ def test_matmul_swiglu_equals_unfused_sequence(agemm, fmt, M, F, K, S):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-def test_grouped_matmul_swiglu_equals_unfused_sequence(agemm, fmt):
+@pytest.mark.parametrize("counts", [[5, 0, 170, 1, 300, 0, 64, 9], [2500, 2100]])
+def test_grouped_matmul_swiglu_equals_unfused_sequence(agemm, fmt, counts):
     import torch.nn.functional as Fn
-    counts, F, K, S = [5, 0, 170, 1, 300, 0, 64, 9], 256, 512, 128
+    F, K, S = 256, 512, 128
     T, E = sum(counts), len(counts)
     g = torch.Generator().manual_seed(77)
     x = recipes.activations(T, K, seed=9200, outlier_frac=0.01, outlier_gain=40.0).cuda()
