@@ -300,6 +300,14 @@ __device__ __forceinline__ void lds_dma16(const void *g, uint32_t lds_wave_base)
                : "memory");
 }
 
+// The same with a wave-uniform base address and a 32-bit byte offset per lane.
+__device__ __forceinline__ void lds_dma16_at(const void *base, uint32_t lane_offset, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_wave_base), "v"(lane_offset), "s"(base)
+               : "memory");
+}
+
 __device__ __forceinline__ void lds_dma4(const void *g, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(lds_wave_base), "v"(g) : "memory");
 }
@@ -487,12 +495,32 @@ __device__ __forceinline__ v8i fp4_operand(uint4 q) {
   return __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1);
 }
 
+// Scheduling pattern of one MXFP4 sub-step: NM MFMAs with NR LDS reads (the next sub-step's operands)
+// spread behind them, the first MFMAs taking the larger shares.
+template <int NM, int NR, int M = 0>
+struct MfmaReadPattern {
+  static __device__ __forceinline__ void apply() {
+    if constexpr (M < NM) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      constexpr int R = (NR + NM - 1 - M) / NM;
+      if constexpr (R > 0) __builtin_amdgcn_sched_group_barrier(0x100, R, 0);
+      MfmaReadPattern<NM, NR, M + 1>::apply();
+    }
+  }
+};
+
 template <int WN, int WM, int NS = 2, int NWM = 2>
 __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
   // waves: 2 along N x NWM along M (wave = n + 2 * m), each with WN x WM accumulator tiles of 32 x 32
   constexpr int BN = 64 * WN, BM = 32 * WM * NWM, NW = 2 * NWM;
-  constexpr int RPI = 16 * NWM;  // rows of 128 code bytes that one load instruction of the workgroup covers
+  // Eight waves (two per SIMD): the first wave of every SIMD requests the whole next stage, the second one
+  // goes straight to its MFMAs, so the matrix pipe works while the requests queue up in the load unit.
+  constexpr bool kLoaderWaves = NWM == 4 && NS == 2;
+  constexpr int NLW = kLoaderWaves ? NW / 2 : NW;  // waves that request the stages
+
+  constexpr int RPI = 8 * NLW;   // rows of 128 code bytes that one load instruction of the requesting waves covers
   static_assert(NS == 2 || (NS == 4 && WN == 2 && WM <= 2 && NWM == 2), "the four-stage ring's wait counts are those of the 128x64 and 128x128 tiles");
+  static_assert(!kLoaderWaves || (BN / 64 <= NLW && BM / 64 <= NLW), "one scale load per operand and requesting wave");
   __shared__ uint4 sW[NS * BN * 8], sX[NS * BM * 8];  // code tiles, NS stages each
   __shared__ uint4 sWs[NS * BN], sXs[NS * BM];        // 16 scale bytes per row (two K steps), NS stages each
   const int tid = threadIdx.x, lane = tid & 63;
@@ -517,28 +545,48 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
   const bool short_last = (p.Kp & 255) != 0;  // then the last step has 4 valid blocks (K' % 256 == 128)
 
   // ---- global -> LDS plan: codes
-  const int ld_row = tid >> 3;                                   // + RPI*i
+  const int ld_row = (tid >> 3) & (RPI - 1);                     // + RPI*i
   const int ld_q = (tid & 7) ^ ((ld_row >> 1) & 7);              // chunk fetched by this lane
-  const uint8_t *wsrc[BN / RPI], *xsrc[BM / RPI];
+  // With requesting waves the addresses are a wave-uniform base (operand + K offset) plus a 32-bit byte
+  // offset per lane (the host sends operands of 4 GiB and more to the four-wave kernels).
+  constexpr int NPW = kLoaderWaves ? 1 : BN / RPI, NPX = kLoaderWaves ? 1 : BM / RPI;
+  constexpr int NOW = kLoaderWaves ? BN / RPI : 1, NOX = kLoaderWaves ? BM / RPI : 1;
+  const uint8_t *wsrc[NPW], *xsrc[NPX];
+  uint32_t wvo[NOW], xvo[NOX];
+  if constexpr (kLoaderWaves) {
 #pragma unroll
-  for (int i = 0; i < BN / RPI; ++i)
-    wsrc[i] = p.b_codes + (size_t)min(n_base + RPI * i + ld_row, p.N - 1) * kbytes + ld_q * 16;
+    for (int i = 0; i < BN / RPI; ++i) wvo[i] = (uint32_t)min(n_base + RPI * i + ld_row, p.N - 1) * (uint32_t)kbytes + ld_q * 16;
 #pragma unroll
-  for (int i = 0; i < BM / RPI; ++i)
-    xsrc[i] = p.a_codes + (size_t)min(m_base + RPI * i + ld_row, p.M - 1) * kbytes + ld_q * 16;
+    for (int i = 0; i < BM / RPI; ++i) xvo[i] = (uint32_t)min(m_base + RPI * i + ld_row, p.M - 1) * (uint32_t)kbytes + ld_q * 16;
+  } else {
+#pragma unroll
+    for (int i = 0; i < BN / RPI; ++i)
+      wsrc[i] = p.b_codes + (size_t)min(n_base + RPI * i + ld_row, p.N - 1) * kbytes + ld_q * 16;
+#pragma unroll
+    for (int i = 0; i < BM / RPI; ++i)
+      xsrc[i] = p.a_codes + (size_t)min(m_base + RPI * i + ld_row, p.M - 1) * kbytes + ld_q * 16;
+  }
   // ---- scales: a lane fetches 16 bytes = the E8M0 bytes of one row for a PAIR of K steps; one
-  // load instruction covers 64 rows.  Instruction j of the weights goes to wave j%4, of the
-  // activations to wave (j+WN)%4.  If the row ends inside the last pair, the 16-byte window is
+  // load instruction covers 64 rows.  Instruction j of the weights goes to wave j%NW, of the
+  // activations to wave (j+BN/64)%NW; with requesting waves, instruction j of either operand to wave j.
+  // If the row ends inside the last pair, the 16-byte window is
   // shifted back to end at the row end (sc_shift bytes; K' % 128 == 0 makes it a multiple of 4).
   const int npairs = (nk + 1) >> 1;
   const int sc_shift = max(0, npairs * 16 - ksc);
-  const uint8_t *wssrc[BN / 64], *xssrc[BM / 64];
+  constexpr int NPS = kLoaderWaves ? 1 : BN / 64, NPT = kLoaderWaves ? 1 : BM / 64;
+  const uint8_t *wssrc[NPS], *xssrc[NPT];
+  uint32_t wsvo = 0, xsvo = 0;
+  if constexpr (kLoaderWaves) {
+    wsvo = (uint32_t)min(n_base + 64 * min(wave, BN / 64 - 1) + lane, p.N - 1) * (uint32_t)ksc;
+    xsvo = (uint32_t)min(m_base + 64 * min(wave, BM / 64 - 1) + lane, p.M - 1) * (uint32_t)ksc;
+  } else {
 #pragma unroll
-  for (int j = 0; j < BN / 64; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
+    for (int j = 0; j < BN / 64; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
 #pragma unroll
-  for (int j = 0; j < BM / 64; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
-  const uint32_t lw0 = (uint32_t)reinterpret_cast<uintptr_t>(sW) + wave * 1024;
-  const uint32_t lx0 = (uint32_t)reinterpret_cast<uintptr_t>(sX) + wave * 1024;
+    for (int j = 0; j < BM / 64; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
+  }
+  const uint32_t lw0 = (uint32_t)reinterpret_cast<uintptr_t>(sW) + (wave % NLW) * 1024;
+  const uint32_t lx0 = (uint32_t)reinterpret_cast<uintptr_t>(sX) + (wave % NLW) * 1024;
   const uint32_t lws0 = (uint32_t)reinterpret_cast<uintptr_t>(sWs);
   const uint32_t lxs0 = (uint32_t)reinterpret_cast<uintptr_t>(sXs);
 
@@ -547,20 +595,35 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
     // a short last step has only chunks 0..3: fetch those twice; the products of the absent blocks
     // are zeroed in compute()
     const bool clip = short_last && kt == nk - 1;
+    if constexpr (kLoaderWaves) {
+      const uint8_t *wb = p.b_codes + kt * 128, *xb = p.a_codes + kt * 128;
+      const uint32_t back = (clip && ld_q >= 4) ? 64u : 0u;
+#pragma unroll
+      for (int i = 0; i < BN / RPI; ++i) lds_dma16_at(wb, wvo[i] - back, lw0 + st * (BN * 128) + i * (RPI * 128));
+#pragma unroll
+      for (int i = 0; i < BM / RPI; ++i) lds_dma16_at(xb, xvo[i] - back, lx0 + st * (BM * 128) + i * (RPI * 128));
+      if ((kt & 1) == 0) {  // scales of steps kt and kt+1
+        const int pair = kt >> 1, sst = pair & (NS - 1);
+        const int soff = pair * 16 - (pair == npairs - 1 ? sc_shift : 0);
+        if (wave < BN / 64) lds_dma16_at(p.b_scales + soff, wsvo, lws0 + sst * (BN * 16) + wave * 1024);
+        if (wave < BM / 64) lds_dma16_at(p.a_scales + soff, xsvo, lxs0 + sst * (BM * 16) + wave * 1024);
+      }
+    } else {
     const int koff = kt * 128 - ((clip && ld_q >= 4) ? 64 : 0);
 #pragma unroll
-    for (int i = 0; i < BN / RPI; ++i) lds_dma16(wsrc[i] + koff, lw0 + st * (BN * 128) + i * (RPI * 128));
+    for (int i = 0; i < NPW; ++i) lds_dma16(wsrc[i] + koff, lw0 + st * (BN * 128) + i * (RPI * 128));
 #pragma unroll
-    for (int i = 0; i < BM / RPI; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * (RPI * 128));
+    for (int i = 0; i < NPX; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * (RPI * 128));
     if ((kt & 1) == 0) {  // scales of steps kt and kt+1
       const int pair = kt >> 1, sst = pair & (NS - 1);
       const int soff = pair * 16 - (pair == npairs - 1 ? sc_shift : 0);
 #pragma unroll
-      for (int j = 0; j < BN / 64; ++j)
+      for (int j = 0; j < NPS; ++j)
         if ((j % NW) == wave) lds_dma16(wssrc[j] + soff, lws0 + sst * (BN * 16) + j * 1024);
 #pragma unroll
-      for (int j = 0; j < BM / 64; ++j)
+      for (int j = 0; j < NPT; ++j)
         if (((j + BN / 64) % NW) == wave) lds_dma16(xssrc[j] + soff, lxs0 + sst * (BM * 16) + j * 1024);
+    }
     }
   };
 
@@ -585,8 +648,8 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   // One K step.  TAIL: the short last step (blocks 4..7 absent): lanes with kh = 1 multiply zeros.
-  // The operand reads of sub-step ks+1 are issued before the MFMAs of sub-step ks (two register
-  // sets), so LDS latency hides behind the matrix pipe.
+  // The operand reads of sub-step ks+1 go out between the MFMAs of sub-step ks (two register sets,
+  // one read behind each of the first MFMAs), so neither their issue nor their latency idles the matrix pipe.
   auto compute = [&](int kt, auto tail) {
     constexpr bool TAIL = decltype(tail)::value;
     const int st = kt & (NS - 1), sst = (kt >> 1) & (NS - 1);
@@ -598,11 +661,12 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
     const int *cxs = reinterpret_cast<const int *>(sXs) + sst * (BM * 4) + sdw;
     int ws[WN], xs[WM];
     uint4 wq[2][WN], xq[2][WM];
-    auto fetch = [&](int ks, int b) {
+    auto fetch = [&](int ks, int b) {  // in the order in which the MFMAs need them
 #pragma unroll
-      for (int i = 0; i < WN; ++i) wq[b][i] = cw[w_rd[ks] + i * 256];
-#pragma unroll
-      for (int j = 0; j < WM; ++j) xq[b][j] = cx[x_rd[ks] + j * 256];
+      for (int t = 0; t < (WN > WM ? WN : WM); ++t) {
+        if (t < WM) xq[b][t] = cx[x_rd[ks] + t * 256];
+        if (t < WN) wq[b][t] = cw[w_rd[ks] + t * 256];
+      }
     };
 #pragma unroll
     for (int i = 0; i < WN; ++i) ws[i] = cws[ws_rd + i * 128];
@@ -612,7 +676,6 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
 #define ARCQ_MX_SUBSTEP(KS)                                                                                   \
   {                                                                                                           \
     if (KS < 3) fetch(KS + 1, (KS + 1) & 1);                                                                  \
-    __builtin_amdgcn_sched_barrier(0);                                                                        \
     v8i wf[WN], xf[WM];                                                                                       \
     _Pragma("unroll") for (int i = 0; i < WN; ++i) {                                                          \
       uint4 q = wq[KS & 1][i];                                                                                \
@@ -627,6 +690,7 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
     _Pragma("unroll") for (int i = 0; i < WN; ++i) _Pragma("unroll") for (int j = 0; j < WM; ++j)             \
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[i], xf[j], acc[i][j], 4, 4, KS, ws[i], \
                                                                      KS, xs[j]);                              \
+    if (KS < 3) MfmaReadPattern<WN * WM, WN + WM>::apply();                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                                        \
   }
     ARCQ_MX_SUBSTEP(0)
@@ -663,12 +727,13 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   };
+  const bool requests = wave < NLW;
 #pragma unroll
   for (int a = 0; a < NS - 1; ++a)
-    if (kt_beg + a < kt_end) issue(kt_beg + a);
+    if (kt_beg + a < kt_end && requests) issue(kt_beg + a);
   for (int kt = kt_beg; kt < nfull; ++kt) {
     wait_step(kt_end - 1 - kt);  // the stage of step kt is complete; everyone is done with the stage of step kt-1
-    if (kt + NS - 1 < kt_end) issue(kt + NS - 1);
+    if (kt + NS - 1 < kt_end && requests) issue(kt + NS - 1);
     compute(kt, std::false_type{});
   }
   if (tail && kt_beg < kt_end) {
@@ -1269,7 +1334,9 @@ int run_gemm(GemmParams p, const GemmPlan &plan, int fmt, float *scratch, hipStr
   if (plan.kernel == 1)
     return fmt == ARCQ_FMT_MXFP4 ? launch_skinny_for<ARCQ_FMT_MXFP4>(p, st) : launch_skinny_for<ARCQ_FMT_NVFP4>(p, st);
   if (fmt == ARCQ_FMT_MXFP4) {
-    switch (plan.kernel) {
+    // the eight-wave kernels address an operand's rows with 32-bit byte offsets from its base
+    const bool wide = (size_t)std::max(p.M, p.N) * (size_t)(p.Kp >> 1) >= ((size_t)1 << 32);
+    switch (wide && plan.kernel == 84 ? 44 : (wide && plan.kernel == 82 ? 42 : plan.kernel)) {
       case 44: return launch_mxfp4_tiled<4, 4>(p, st);
       case 84: return launch_mxfp4_tiled<4, 2, 2, 4>(p, st);  // 256x256 tile, eight waves of 128x64
       case 82: return launch_mxfp4_tiled<4, 1, 2, 4>(p, st);  // 256x128 tile, eight waves of 128x32
