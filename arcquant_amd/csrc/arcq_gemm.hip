@@ -1256,10 +1256,12 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
   } else if (split_env == 0 && force < 0 && M > 64 && M <= 512) {
     // Up to a few hundred rows on a narrow layer: the larger tiles leave most CUs without a workgroup,
     // and a workgroup's time is its number of K steps times the memory latency, whatever M is.  As
-    // many 128x64 tiles x K slices as there are CUs; two slices anyway when K is long.
+    // many 128x64 tiles x K slices as there are CUs when K is long (NVFP4, whose workgroups fit two to a CU:
+    // two slices anyway; the MXFP4 ring kernel has one workgroup per CU, and a second round costs more than
+    // the slices save: down projection at M = 512, 38 us uncut against 49 us in two slices).
     const long tiles21 = (long)((M + 63) / 64) * ((N + 127) / 128);
     if (tiles21 <= 256) {
-      int sl = Kp >= 8192 ? std::max(2, (int)(256 / tiles21)) : 1;
+      int sl = Kp >= 8192 ? (fmt == ARCQ_FMT_MXFP4 ? (int)(256 / tiles21) : std::max(2, (int)(256 / tiles21))) : 1;
       if (fmt == ARCQ_FMT_NVFP4 && Kp < 8192) sl = (int)(256 / tiles21);  // no ring there: slices hide the latency
       if (sl >= 2) split = std::min(sl, 8);
       else one_round_21 = true;
