@@ -1305,7 +1305,9 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
                                               : (M <= 128 ? 21
                                                           : (M < 512 ? 22
                                                                      : (c44 < c42 && c44 < c22 ? 84 : (c42 <= c22 ? 82 : 22)))));
-    plan.kernel = force > 1 ? force : pick;
+    const bool known = force == 44 || force == 84 || force == 82 || force == 42 || force == 224 || force == 22 ||
+                       force == 214 || force == 21;
+    plan.kernel = known ? force : pick;
     return plan;
   }
   if (fmt == ARCQ_FMT_NVFP4 && force != 0 && tiled_ok) {
@@ -1314,7 +1316,8 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
     // against 74 us with 256x128 tiles), so the next smaller tile that still fills it
     const long t44 = (long)((M + 255) / 256) * ((N + 255) / 256), t42 = (long)((M + 127) / 128) * ((N + 255) / 256);
     const int pick = t44 >= 192 ? 44 : (M > 128 && !one_round_21 ? (t42 >= 192 ? 42 : 22) : 21);
-    plan.kernel = force > 1 ? force : pick;
+    const bool known = force == 44 || force == 84 || force == 42 || force == 22 || force == 21;
+    plan.kernel = known ? force : pick;  // a forced kernel that NVFP4 does not have is ignored
     return plan;
   }
   plan.kernel = 0;
@@ -1359,6 +1362,8 @@ int run_gemm(GemmParams p, const GemmPlan &plan, int fmt, float *scratch, hipStr
       default: break;
     }
   }
+  // the direct kernels know neither the fused SwiGLU epilogue (half as many output columns) nor expert segments
+  if (p.swiglu || p.seg) return ARCQ_ERR_SHAPE;
   const dim3 grid((p.N + kWgN - 1) / kWgN, (p.M + kWgM - 1) / kWgM);
   if (fmt == ARCQ_FMT_MXFP4)
     hipLaunchKernelGGL(gemm_mxfp4_direct, grid, dim3(256), 0, st, p);
@@ -1574,8 +1579,9 @@ extern "C" int arcq_matmul_swiglu(const void *a_codes, const void *a_scales, con
   p.swiglu = 1;
   p.absmax_bits = reinterpret_cast<uint32_t *>(d_absmax);
   GemmPlan plan = plan_gemm(M, N, Kp, fmt, true);
-  const bool tiled = plan.slices == 1 && (plan.kernel == 82 || plan.kernel == 84 || plan.kernel == 44 || plan.kernel == 42 || plan.kernel == 22 ||
-                                          plan.kernel == 21 || plan.kernel == 224 || plan.kernel == 214);
+  const int id = plan.kernel;  // (a kernel forced through the environment may not exist for this format)
+  const bool tiled = plan.slices == 1 && (id == 84 || id == 44 || id == 42 || id == 22 || id == 21 ||
+                                          (fmt == ARCQ_FMT_MXFP4 && (id == 82 || id == 224 || id == 214)));
   if (!tiled) {  // the decode-batch kernels and split-K have no fused epilogue: a small tile instead
     plan = GemmPlan();
     plan.kernel = M > 64 ? 22 : 21;

@@ -253,3 +253,36 @@ def test_grouped_matmul_swiglu_equals_unfused_sequence(agemm, fmt, counts):
         rows = want[segc[e]:segc[e + 1]]
         w = float(rows.abs().max().float() / torch.full((), 2688.0, device="cuda")) if rows.numel() else 0.0
         assert float(ts[e]) == (w if w != 0.0 else 1.0), e
+
+
+def test_forced_kernel_unknown_to_the_format_is_ignored():
+    """ARCQ_GEMM_KERNEL names a tile kernel by number; NVFP4 has no 256x128 eight-wave kernel (82).  The fused
+    SwiGLU GEMM must then take a kernel it has, not fall through to the direct kernel, which writes all N
+    output columns.  The knob is read once per process: a child process with it set."""
+    import os
+    import subprocess
+    import sys
+    code = r"""
+import sys, torch
+sys.path.insert(0, 'tests')
+import recipes
+import torch.nn.functional as Fn
+from arcquant_amd import agemm
+M, F, K, S = 300, 256, 512, 128
+x = recipes.activations(M, K, seed=1).cuda()
+idx = torch.randperm(K, generator=torch.Generator().manual_seed(3)).to(torch.int16).cuda()
+wg = recipes.weights(F, K, seed=2, std=0.05).cuda(); wu = recipes.weights(F, K, seed=4, std=0.05).cuda()
+for fmt in ("NVFP4", "MXFP4"):
+    a, sfa = agemm.reorder_quantize_x(x, idx, S, fmt=fmt)
+    b_cat, sfb_cat = agemm.reorder_quantize_w(torch.cat([wg, wu]), idx, S, fmt=fmt)
+    b_il, sfb_il = agemm.reorder_quantize_w(agemm.interleave_gate_up(wg, wu), idx, S, fmt=fmt)
+    h = agemm.matmul(a, b_cat, sfa, sfb_cat, 1.0, fmt=fmt)
+    got = agemm.matmul_swiglu(a, b_il, sfa, sfb_il, 1.0, fmt=fmt)
+    torch.cuda.synchronize()
+    assert torch.equal(got, Fn.silu(h[:, :F]) * h[:, F:]), fmt
+print("OK")
+"""
+    env = dict(os.environ, ARCQ_GEMM_KERNEL="82")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "OK" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
