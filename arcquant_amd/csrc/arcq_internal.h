@@ -38,7 +38,8 @@ constexpr size_t kWorkspaceBytes[kWsKinds] = {256, 32u << 20, 8u << 20};
 void *stream_workspace(int kind, hipStream_t stream, int *status);
 
 // Overrides for tuning runs, read from the environment once, when the library is first used:
-//   ARCQ_GEMM_KERNEL=<WN><WM>   force a GEMM tile (84 = 256x256 as eight waves, 44, 42, 22, 21; 214 / 224 = four-stage ring; 1 = skinny, 0 = direct)
+//   ARCQ_GEMM_KERNEL=<WN><WM>   force a GEMM tile (84 / 82 = 256x256 / 256x128 as eight waves, 44, 42, 22, 21; 214 / 224 = four-stage
+//                               ring; 1 = skinny, 0 = direct); a number the format has no kernel for is ignored
 //   ARCQ_GEMM_SPLITK=<slices>   force split-K for M <= 512 (1 = never split)
 //   ARCQ_QUANT_GRID=<n>         workgroups of the row quantizers
 //   ARCQ_QUANT_KERNEL=<1|2>     1 = never, 2 = always take the wave-per-row quantizer where it has an instance

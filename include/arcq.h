@@ -182,7 +182,7 @@ int arcq_matmul_add(const void *a_codes, const void *a_scales, const void *b_cod
  * buffer, and the call contains no allocation of any kind.
  *   - A problem whose plan needs more than arcq_matmul_noalloc_limit() bytes of partial tiles
  *     (arcq_matmul_scratch_bytes tells, 0 = none needed) is refused with ARCQ_ERR_WORKSPACE and nothing is
- *     launched: e.g. the 4096 x 14336 down projection at 512 rows (two K slices, 16 MiB).  Every decode batch
+ *     launched: e.g. the NVFP4 4096 x 14336 down projection at 512 rows (two K slices, 16 MiB).  Every decode batch
  *     (M <= 64) of the Llama-3-8B shapes fits.
  *   - All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams,
  *     two threads) race.  The array keeps the last call's contents; every word a call reads back it has

@@ -66,9 +66,11 @@ def test_noalloc_without_scratch_and_beyond_the_limit(L):
     rc1, got = call(L.arcq_matmul_noalloc, ops, M, N, K + S, 1)
     torch.cuda.synchronize()
     assert rc0 == 0 and rc1 == 0 and torch.equal(got, want)
-    # down projection at 512 rows: two slices of 512 x 4096 fp32 = 16 MiB, beyond the array -> refused, nothing launched
+    # NVFP4 down projection at 512 rows: two slices of 512 x 4096 fp32 = 16 MiB, beyond the array -> refused,
+    # nothing launched (MXFP4 does not cut K there: its plan needs no scratch)
     M, N, Kp = 512, 4096, 14592
-    assert L.arcq_matmul_scratch_bytes(M, N, Kp, 1) > L.arcq_matmul_noalloc_limit()
+    assert L.arcq_matmul_scratch_bytes(M, N, Kp, 1) == 0
+    assert L.arcq_matmul_scratch_bytes(M, N, Kp, 0) > L.arcq_matmul_noalloc_limit()
     ok = ctypes.c_void_p(0x1000)                                   # never dereferenced: the call returns first
-    assert L.arcq_matmul_noalloc(ok, ok, ok, ok, M, N, Kp, 1, 1.0, None, None, ok, None) == 7
+    assert L.arcq_matmul_noalloc(ok, ok, ok, ok, M, N, Kp, 0, 1.0, None, None, ok, None) == 7
     assert b"scratch" in L.arcq_status_string(7)
