@@ -1530,12 +1530,17 @@ int grouped_matmul_impl(const void *a_codes, const void *a_scales, const void *b
   p.absmax_bits = reinterpret_cast<uint32_t *>(d_absmax);
   // Tile from the rows an average segment holds (the real counts live on the device).  The larger tiles are
   // faster per flop, but every segment ends in a partly empty tile of rows and skewed routing leaves some
-  // segments far below the average: on 8192 rows over 8 segments of 195..3120 rows the 128x128 tile beat
-  // 256x128 and 256x256 for both formats (two GEMMs: 1.82 / 1.99 / 1.93 ms MXFP4, 3.80 / 3.87 / 3.87 NVFP4).
+  // segments far below the average.  Measured on 8 segments of skewed sizes (a Mixtral block's two GEMMs and
+  // what runs between them): NVFP4, 8192 rows of 195..3120 per segment: 128x128 tiles 3.51 ms, 256x128 3.70,
+  // 256x256 3.86-3.96; MXFP4 with the eight-wave 256x256 kernel against 128x128 tiles: 0.66 / 0.74 ms at 2048
+  // rows, 1.00 / 1.03 at 4096, 1.18 / 1.32 at 6144, 1.52 / 1.65 at 8192.
   const int avg = M / n_seg;
   GemmPlan plan;
   const int force = tuning().gemm_kernel;
-  plan.kernel = avg >= 2048 ? (fmt == ARCQ_FMT_MXFP4 ? 84 : 44) : (avg >= 96 ? 22 : 21);
+  if (fmt == ARCQ_FMT_MXFP4)
+    plan.kernel = avg >= 256 ? 84 : (avg >= 96 ? 22 : 21);
+  else
+    plan.kernel = avg >= 2048 ? 44 : (avg >= 96 ? 22 : 21);
   if (force == 84 || force == 44 || force == 42 || force == 22 || force == 21) plan.kernel = force;
   return run_gemm(p, plan, fmt, nullptr, static_cast<hipStream_t>(stream));
 }
