@@ -95,9 +95,7 @@ __device__ __forceinline__ bool enter_segment(GemmParams &p, int &lin) {
 
 // two bf16 pairs + two bf16 pairs, each sum rounded to bf16
 __device__ __forceinline__ uint32_t add_bf16_pair(uint32_t a, uint32_t b) {
-  const uint32_t lo = f32_to_bf16_bits(bf16_bits_to_f32(a & 0xffffu) + bf16_bits_to_f32(b & 0xffffu));
-  const uint32_t hi = f32_to_bf16_bits(bf16_bits_to_f32(a >> 16) + bf16_bits_to_f32(b >> 16));
-  return lo | (hi << 16);
+  return pack_bf16_rne(u2f(a << 16) + u2f(b << 16), u2f(a & 0xffff0000u) + u2f(b & 0xffff0000u));
 }
 __device__ __forceinline__ uint2 add_bf16_x4(uint2 a, uint2 b) {
   return make_uint2(add_bf16_pair(a.x, b.x), add_bf16_pair(a.y, b.y));
@@ -122,10 +120,8 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, const v16f &acc,
     uint16_t *crow = p.c + (size_t)m * p.N + n0 + 4 * (lane >> 5);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      uint32_t h[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) h[j] = f32_to_bf16_bits(acc[4 * q + j] * alpha);
-      uint2 v = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+      uint2 v = make_uint2(pack_bf16_rne(acc[4 * q] * alpha, acc[4 * q + 1] * alpha),
+                           pack_bf16_rne(acc[4 * q + 2] * alpha, acc[4 * q + 3] * alpha));
       if (p.residual) v = add_bf16_x4(v, *reinterpret_cast<const uint2 *>(p.residual + (crow - p.c) + 8 * q));
       *reinterpret_cast<uint2 *>(crow + 8 * q) = v;
     }
@@ -374,12 +370,11 @@ __device__ __forceinline__ void store_workgroup_tile(const GemmParams &p, v16f (
         const int sw = (m & (LPR - 1)) << 1;          // even: keeps 8-byte chunk pairs adjacent
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          uint32_t h[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) h[e] = f32_to_bf16_bits(acc[i][j][4 * q + e] * alpha);
+          const v16f &a = acc[i][j];                  // the hardware's round-to-nearest-even convert
           const int c = 8 * i + 2 * q + kh;           // 8-byte chunk of the row
           *reinterpret_cast<uint2 *>(region + m * RB + ((c ^ sw) << 3)) =
-              make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+              make_uint2(pack_bf16_rne(a[4 * q] * alpha, a[4 * q + 1] * alpha),
+                         pack_bf16_rne(a[4 * q + 2] * alpha, a[4 * q + 3] * alpha));
         }
       }
     const int rr = lane / LPR, t = lane % LPR;
@@ -1009,8 +1004,7 @@ __device__ __forceinline__ void skinny_reduce_store(const GemmParams &p, v4f (&a
       if (m >= p.M) continue;
       uint16_t *dst = p.c + (size_t)m * p.N + n0;
       if (n0 + 3 < p.N && (p.N & 3) == 0) {
-        const uint32_t lo = f32_to_bf16_bits(t[0] * alpha) | (f32_to_bf16_bits(t[1] * alpha) << 16);
-        const uint32_t hi = f32_to_bf16_bits(t[2] * alpha) | (f32_to_bf16_bits(t[3] * alpha) << 16);
+        const uint32_t lo = pack_bf16_rne(t[0] * alpha, t[1] * alpha), hi = pack_bf16_rne(t[2] * alpha, t[3] * alpha);
         uint2 v = make_uint2(lo, hi);
         if (p.residual) v = add_bf16_x4(v, *reinterpret_cast<const uint2 *>(p.residual + (dst - p.c)));
         *reinterpret_cast<uint2 *>(dst) = v;
@@ -1212,8 +1206,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(GemmParams p) {
       const float4 u = reinterpret_cast<const float4 *>(p.partial + (size_t)k * plane)[i];
       t.x += u.x, t.y += u.y, t.z += u.z, t.w += u.w;
     }
-    const uint32_t lo = f32_to_bf16_bits(t.x * alpha) | (f32_to_bf16_bits(t.y * alpha) << 16);
-    const uint32_t hi = f32_to_bf16_bits(t.z * alpha) | (f32_to_bf16_bits(t.w * alpha) << 16);
+    const uint32_t lo = pack_bf16_rne(t.x * alpha, t.y * alpha), hi = pack_bf16_rne(t.z * alpha, t.w * alpha);
     uint2 v = make_uint2(lo, hi);
     if (p.residual) v = add_bf16_x4(v, reinterpret_cast<const uint2 *>(p.residual)[i]);
     reinterpret_cast<uint2 *>(p.c)[i] = v;
