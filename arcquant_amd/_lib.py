@@ -80,6 +80,10 @@ def lib() -> ctypes.CDLL:
         getattr(L, name).restype = i
     L.arcq_moe_combine.argtypes = [vp, vp, vp, i, i, i, i, vp, vp]
     L.arcq_moe_combine.restype = i
+    L.arcq_moe_route.argtypes = [vp, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+    L.arcq_moe_route.restype = i
+    L.arcq_moe_route_workspace_bytes.argtypes = [i, i]
+    L.arcq_moe_route_workspace_bytes.restype = sz
     for name in ("arcq_grouped_reorder_quantize_x", "arcq_grouped_swiglu_quantize_x", "arcq_grouped_tensor_scale",
                  "arcq_grouped_matmul"):
         getattr(L, name).restype = i

@@ -33,7 +33,7 @@ from ._lib import FORMATS, ArcqError  # noqa: F401
 __all__ = ["matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "init_kv_i4", "append_kv_i4",
            "batch_decode_i4", "swiglu_quantize_x", "tensor_scale", "prepare_stream", "dequantize", "check_index",
            "unpack_codes", "scale_values", "grouped_tensor_scale", "grouped_reorder_quantize_x",
-           "grouped_swiglu_quantize_x", "grouped_matmul", "moe_combine", "matmul_swiglu",
+           "grouped_swiglu_quantize_x", "grouped_matmul", "moe_route", "moe_combine", "matmul_swiglu",
            "grouped_matmul_swiglu", "interleave_gate_up"]
 
 
@@ -464,6 +464,36 @@ def grouped_matmul_swiglu(A, B, SFA, SFB, seg, scale_a=None, scale_b=None, *, fm
     if tensor_scale:
         return T, _absmax_to_scales(amax, 2688.0)
     return T
+
+
+def moe_route(router_logits, top_k):
+    """Routing of a mixture-of-experts block in two launches (model/qMixtralLayer.py:441-452 and the bookkeeping
+    of its loop over experts): softmax in fp32, top-k, weights divided by their sum, bf16.  Returns
+    (sel int32 [T, k], weight bf16 [T, k], seg_offsets int32 [E+1], position int64 [T*k], token_of_row int32
+    [T*k], weight_of_row bf16 [T*k]); rows of one expert keep ascending (token, slot) order.  Among equal
+    probabilities the lower expert number is taken."""
+    if router_logits.dim() != 2 or router_logits.dtype not in (torch.bfloat16, torch.float32) or not router_logits.is_cuda:
+        raise RuntimeError("moe_route: router_logits must be a bf16 or fp32 [tokens, experts] tensor on the GPU")
+    router_logits = router_logits.contiguous()
+    T, E = router_logits.shape
+    if not 1 <= top_k <= min(8, E) or E > 64:
+        raise RuntimeError(f"Value error in moe_route: experts={E}, top_k={top_k}")
+    dev = router_logits.device
+    sel = torch.empty((T, top_k), dtype=torch.int32, device=dev)
+    weight = torch.empty((T, top_k), dtype=torch.bfloat16, device=dev)
+    seg = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    position = torch.empty(T * top_k, dtype=torch.int64, device=dev)
+    tok = torch.empty(T * top_k, dtype=torch.int32, device=dev)
+    ws = torch.empty(T * top_k, dtype=torch.bfloat16, device=dev)
+    L = _lib.lib()
+    nbytes = L.arcq_moe_route_workspace_bytes(T, E)
+    work = torch.empty(max(nbytes, 4), dtype=torch.uint8, device=dev)
+    with _on_device(router_logits):
+        rc = L.arcq_moe_route(router_logits.data_ptr(), int(router_logits.dtype == torch.float32), T, E, top_k,
+                              sel.data_ptr(), weight.data_ptr(), seg.data_ptr(), position.data_ptr(), tok.data_ptr(),
+                              ws.data_ptr(), work.data_ptr(), work.numel(), _stream(router_logits))
+    _lib.check(rc, "arcq_moe_route")
+    return sel, weight, seg, position, tok, ws
 
 
 def moe_combine(y, position, weight, tokens, top_k):

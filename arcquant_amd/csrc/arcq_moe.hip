@@ -70,8 +70,188 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t *y, con
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Routing (model/qMixtralLayer.py:441-452: softmax over the experts in fp32, top-k, the k weights divided by
+// their sum and cast to the activations' type; :456-471 then walks the experts and the tokens routed to each).
+// Two launches replace a dozen of torch's: per token the choice and its weights, per (token, slot) pair its row
+// in the expert-sorted order (pairs of one expert in ascending pair number, as a stable sort by expert gives),
+// the expert segments, and the sorted views of token number and weight the grouped launches read.
+//
+// Arithmetic follows torch's on this device so that the weights come out as the same bits: maximum and sum of
+// exp(l - max) as the butterfly over the next power of two that its warp softmax forms (padding adds zeros),
+// exp(l - max) / sum, top-k weights divided by their sum left to right (exact for k = 2, the Mixtral case).
+// Equal probabilities: the lower expert number wins (torch.topk leaves the choice among equals unspecified).
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaxExperts = 64;
+constexpr int kRouteThreads = 256;
+
+template <bool F32, int P>  // P: the power of two the experts are padded to
+__global__ __launch_bounds__(kRouteThreads) void moe_route_choose_kernel(const void *logits, int T, int E, int top_k, int *sel,
+                                                                         uint16_t *w, int64_t *position, int *hist) {
+  __shared__ int cnt[kRouteThreads / 64][kMaxExperts];
+  const int t = blockIdx.x * kRouteThreads + threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const bool live = t < T;
+  float prob[P];
+  int my[kMaxTopK];
+  float mw[kMaxTopK];
+#pragma unroll
+  for (int j = 0; j < kMaxTopK; ++j) { my[j] = -1; mw[j] = 0.0f; }
+  if (live) {
+    float v[P];
+#pragma unroll
+    for (int e = 0; e < P; ++e) {
+      float x = -__builtin_inff();
+      if (e < E)
+        x = F32 ? static_cast<const float *>(logits)[(size_t)t * E + e]
+                : bf16_bits_to_f32(static_cast<const uint16_t *>(logits)[(size_t)t * E + e]);
+      v[e] = x;
+    }
+    float mx = v[0];
+#pragma unroll
+    for (int e = 1; e < P; ++e) mx = fmaxf(mx, v[e]);  // the padding is -inf
+    float red[P];
+#pragma unroll
+    for (int e = 0; e < P; ++e) {
+      prob[e] = e < E ? expf(v[e] - mx) : 0.0f;
+      red[e] = prob[e];
+    }
+#pragma unroll
+    for (int off = P >> 1; off > 0; off >>= 1) {  // lane i of the butterfly: red[i] + red[i ^ off]
+      float nxt[P];
+#pragma unroll
+      for (int e = 0; e < P; ++e) nxt[e] = red[e] + red[e ^ off];
+#pragma unroll
+      for (int e = 0; e < P; ++e) red[e] = nxt[e];
+    }
+    const float sum = red[0];
+#pragma unroll
+    for (int e = 0; e < P; ++e) prob[e] = e < E ? prob[e] / sum : -1.0f;
+    // top-k: k passes over the probabilities, the largest not yet taken, ties to the lower expert number
+    float tot = 0.0f;
+    for (int j = 0; j < top_k; ++j) {
+      int best = -1;
+      float bv = -1.0f;
+#pragma unroll
+      for (int e = 0; e < P; ++e) {
+        bool taken = false;
+#pragma unroll
+        for (int q = 0; q < kMaxTopK; ++q) taken |= q < j && my[q] == e;
+        if (e < E && !taken && prob[e] > bv) { bv = prob[e]; best = e; }
+      }
+      my[j] = best;
+      mw[j] = bv;
+      tot = j == 0 ? bv : tot + bv;
+    }
+    for (int j = 0; j < top_k; ++j) {
+      sel[(size_t)t * top_k + j] = my[j];
+      w[(size_t)t * top_k + j] = (uint16_t)f32_to_bf16_bits(mw[j] / tot);
+    }
+  }
+  // rank of every pair among the pairs of its expert inside this workgroup, in pair order
+  int rank[kMaxTopK];
+#pragma unroll
+  for (int j = 0; j < kMaxTopK; ++j) rank[j] = 0;
+  const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  for (int e = 0; e < E; ++e) {
+    int wave_cnt = 0, before_me = 0;
+    for (int j = 0; j < top_k; ++j) {
+      const unsigned long long m = __builtin_amdgcn_ballot_w64(live && my[j] == e);
+      wave_cnt += __builtin_popcountll(m);
+      before_me += __builtin_popcountll(m & below);
+    }
+    for (int j = 0; j < top_k; ++j)
+      if (my[j] == e) rank[j] = before_me;  // a token takes an expert once: no earlier slot of its own to count
+    if (lane == 0) cnt[wave][e] = wave_cnt;
+  }
+  __syncthreads();
+  if (live)
+    for (int j = 0; j < top_k; ++j) {
+      int base = 0;
+      for (int q = 0; q < wave; ++q) base += cnt[q][my[j]];
+      position[(size_t)t * top_k + j] = base + rank[j];  // finished by the second launch
+    }
+  if (threadIdx.x < E) {
+    int tot = 0;
+    for (int q = 0; q < kRouteThreads / 64; ++q) tot += cnt[q][threadIdx.x];
+    hist[(size_t)blockIdx.x * E + threadIdx.x] = tot;
+  }
+}
+
+__global__ __launch_bounds__(kRouteThreads) void moe_route_place_kernel(int T, int E, int top_k, const int *sel, const uint16_t *w,
+                                                                        const int *hist, int64_t *position, int *seg, int *tok,
+                                                                        uint16_t *ws) {
+  __shared__ int start[kMaxExperts];  // first sorted row of this workgroup's pairs of expert e
+  if (threadIdx.x < E) {
+    const int e = threadIdx.x;
+    int before = 0;  // pairs of experts below e, plus those of e in earlier workgroups
+    for (int b = 0; b < (int)gridDim.x; ++b)
+      for (int q = 0; q < e; ++q) before += hist[(size_t)b * E + q];
+    int seg_e = before;
+    for (int b = 0; b < (int)blockIdx.x; ++b) before += hist[(size_t)b * E + e];
+    start[e] = before;
+    if (blockIdx.x == 0) {
+      seg[e] = seg_e;
+      if (e == E - 1) {
+        int all = seg_e;
+        for (int b = 0; b < (int)gridDim.x; ++b) all += hist[(size_t)b * E + e];
+        seg[E] = all;
+      }
+    }
+  }
+  __syncthreads();
+  const int t = blockIdx.x * kRouteThreads + threadIdx.x;
+  if (t >= T) return;
+  for (int j = 0; j < top_k; ++j) {
+    const size_t pair = (size_t)t * top_k + j;
+    const int64_t pos = start[sel[pair]] + position[pair];
+    position[pair] = pos;
+    tok[pos] = t;
+    ws[pos] = w[pair];
+  }
+}
+
 }  // namespace
 }  // namespace arcq
+
+extern "C" size_t arcq_moe_route_workspace_bytes(int tokens, int experts) {
+  if (tokens < 0 || experts < 1) return 0;
+  return (size_t)((tokens + arcq::kRouteThreads - 1) / arcq::kRouteThreads) * (size_t)experts * sizeof(int);
+}
+
+extern "C" int arcq_moe_route(const void *logits, int logits_f32, int tokens, int experts, int top_k, int *sel, void *weight,
+                              int *seg_offsets, int64_t *position, int *token_of_row, void *weight_of_row, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+  using namespace arcq;
+  if (tokens < 0 || experts < 1 || experts > kMaxExperts || top_k < 1 || top_k > kMaxTopK || top_k > experts)
+    return ARCQ_ERR_SHAPE;
+  if (!seg_offsets) return ARCQ_ERR_NULL;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!logits || !sel || !weight || !position || !token_of_row || !weight_of_row || !workspace) return ARCQ_ERR_NULL;
+  const int blocks = tokens == 0 ? 1 : (tokens + kRouteThreads - 1) / kRouteThreads;
+  if (workspace_bytes < (size_t)blocks * experts * sizeof(int)) return ARCQ_ERR_WORKSPACE;
+  int *hist = static_cast<int *>(workspace);
+#define ARCQ_ROUTE(PP)                                                                                                      \
+  if (logits_f32)                                                                                                          \
+    hipLaunchKernelGGL((moe_route_choose_kernel<true, PP>), dim3(blocks), dim3(kRouteThreads), 0, st, logits, tokens, experts, \
+                       top_k, sel, static_cast<uint16_t *>(weight), position, hist);                                      \
+  else                                                                                                                     \
+    hipLaunchKernelGGL((moe_route_choose_kernel<false, PP>), dim3(blocks), dim3(kRouteThreads), 0, st, logits, tokens, experts, \
+                       top_k, sel, static_cast<uint16_t *>(weight), position, hist);
+  if (experts <= 2) { ARCQ_ROUTE(2) }
+  else if (experts <= 4) { ARCQ_ROUTE(4) }
+  else if (experts <= 8) { ARCQ_ROUTE(8) }
+  else if (experts <= 16) { ARCQ_ROUTE(16) }
+  else if (experts <= 32) { ARCQ_ROUTE(32) }
+  else { ARCQ_ROUTE(64) }
+#undef ARCQ_ROUTE
+  ARCQ_HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(moe_route_place_kernel, dim3(blocks), dim3(kRouteThreads), 0, st, tokens, experts, top_k, sel,
+                     static_cast<const uint16_t *>(weight), hist, position, seg_offsets, token_of_row,
+                     static_cast<uint16_t *>(weight_of_row));
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
 
 extern "C" int arcq_moe_combine(const void *y, const int64_t *position, const void *weight, int tokens, int H, int top_k,
                                 int pairs, void *out, void *stream) {

@@ -619,23 +619,33 @@ class MixtralSparseMoeBlock(nn.Module):
         x = hidden_states.reshape(-1, hid)
         if router_logits is None:
             router_logits = self.gate(x)
-        w = F.softmax(router_logits, dim=1, dtype=torch.float)
-        w, sel = torch.topk(w, self.top_k, dim=-1)
-        w = (w / w.sum(dim=-1, keepdim=True)).to(x.dtype)
-        # (token, slot) pairs sorted by expert: one contiguous run of rows per expert
-        flat_e = sel.reshape(-1)
-        order = torch.argsort(flat_e, stable=True)
-        tok = order // self.top_k
+        fused_route = (x.dtype == torch.bfloat16 and self.num_experts <= 64 and self.top_k <= 8
+                       and router_logits.dtype in (torch.bfloat16, torch.float32))
+        if fused_route:
+            # softmax, top-k, normalised weights and the expert-sorted bookkeeping in two launches
+            sel, w, seg, position, tok, ws = agemm.moe_route(router_logits, self.top_k)
+            flat_e = sel.reshape(-1)
+        else:
+            w = F.softmax(router_logits, dim=1, dtype=torch.float)
+            w, sel = torch.topk(w, self.top_k, dim=-1)
+            w = (w / w.sum(dim=-1, keepdim=True)).to(x.dtype)
+            # (token, slot) pairs sorted by expert: one contiguous run of rows per expert
+            flat_e = sel.reshape(-1)
+            order = torch.argsort(flat_e, stable=True)
+            tok = order // self.top_k
+            ws = w.reshape(-1).index_select(0, order)
+            seg = position = None
         xs = x.index_select(0, tok)
-        ws = w.reshape(-1).index_select(0, order)
         if self.grouped:
-            counts = (flat_e[:, None] == self._expert_ids[None, :]).sum(0)      # on the device: no read-back
-            seg = torch.zeros(self.num_experts + 1, dtype=torch.int32, device=x.device)
-            seg[1:] = torch.cumsum(counts, 0)
+            if seg is None:
+                counts = (flat_e[:, None] == self._expert_ids[None, :]).sum(0)      # on the device: no read-back
+                seg = torch.zeros(self.num_experts + 1, dtype=torch.int32, device=x.device)
+                seg[1:] = torch.cumsum(counts, 0)
             y = self._experts_grouped(xs, seg)
             if hid % 8 == 0 and self.top_k <= 8:
-                position = torch.empty_like(order)
-                position[order] = self._pair_ids(order.numel(), x.device)        # inverse of the sort
+                if position is None:
+                    position = torch.empty_like(order)
+                    position[order] = self._pair_ids(order.numel(), x.device)        # inverse of the sort
                 return agemm.moe_combine(y, position, ws.contiguous(), x.shape[0], self.top_k).reshape(bsz, q_len, hid), \
                     router_logits
             out = torch.zeros_like(x)

@@ -261,6 +261,30 @@ int arcq_matmul_swiglu(const void *a_codes, const void *a_scales, const void *b_
 int arcq_scales_from_absmax(float *d_values, int n, float divisor, void *stream);
 
 /*
+ * Routing of a mixture-of-experts block (model/qMixtralLayer.py:441-452: softmax over the experts in fp32,
+ * top-k, the k weights divided by their sum and cast to bf16; :456-471 then visits expert after expert and the
+ * tokens routed to it).  Two launches, nothing read back: besides each token's choice the call writes what the
+ * grouped launches take -- the expert segments, and for every row of the expert-sorted order its token and its
+ * weight (pairs of one expert in ascending (token, slot) order, as a stable sort by expert number gives).
+ * The arithmetic is torch's on this device (its warp softmax's summation order, exp(l - max) / sum, the top-k
+ * weights divided by their sum left to right), so the weights are the same bits for top_k = 2; among equal
+ * probabilities the lower expert number is taken (torch.topk leaves that choice unspecified).
+ *   logits        [tokens, experts] bf16, or fp32 if logits_f32
+ *   sel           int32 [tokens * top_k]   expert of (token, slot), slots in descending probability
+ *   weight        bf16  [tokens * top_k]   normalised router weight of (token, slot)
+ *   seg_offsets   int32 [experts + 1]      rows seg[e] .. seg[e+1]-1 of the sorted order belong to expert e
+ *   position      int64 [tokens * top_k]   sorted row of (token, slot) (what arcq_moe_combine takes)
+ *   token_of_row  int32 [tokens * top_k]   token whose activations sorted row r reads
+ *   weight_of_row bf16  [tokens * top_k]   router weight of sorted row r
+ *   workspace     arcq_moe_route_workspace_bytes(tokens, experts) bytes of device memory, contents irrelevant
+ * experts <= 64, top_k <= 8 and <= experts.
+ */
+size_t arcq_moe_route_workspace_bytes(int tokens, int experts);
+int arcq_moe_route(const void *logits, int logits_f32, int tokens, int experts, int top_k, int *sel, void *weight,
+                   int *seg_offsets, int64_t *position, int *token_of_row, void *weight_of_row, void *workspace,
+                   size_t workspace_bytes, void *stream);
+
+/*
  * Last step of a mixture-of-experts block: out[t] = sum over token t's experts, in ascending expert number, of
  * bf16(y[row] * weight[row]), every partial sum rounded to bf16 -- what model/qMixtralLayer.py:466-471 gets
  * from `expert(x) * routing_weights[...]` followed by final_hidden_states.index_add_ per expert.  One launch,

@@ -102,5 +102,12 @@ def test_grouped_entry_points_reject_bad_arguments():
     assert mc(ok, ok, ok, 8, 4096, 9, 72, ok, None) == 2                                      # top_k > 8
     assert mc(ok, None, ok, 8, 4096, 2, 16, ok, None) == 1
     assert mc(ok, ok, ok, 0, 4096, 2, 0, ok, None) == 0
+    mr = L.arcq_moe_route
+    assert L.arcq_moe_route_workspace_bytes(4096, 8) == 16 * 8 * 4
+    assert mr(ok, 0, 16, 65, 2, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None) == 2               # more than 64 experts
+    assert mr(ok, 0, 16, 8, 9, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None) == 2                # top_k > 8
+    assert mr(ok, 0, 16, 4, 5, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None) == 2                # top_k > experts
+    assert mr(None, 0, 16, 8, 2, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None) == 1
+    assert mr(ok, 0, 4096, 8, 2, ok, ok, ok, ok, ok, ok, ok, 16, None) == 7                   # workspace too small
     assert L.arcq_stream_probe_variants() >= 2
     assert L.arcq_stream_probe_variant(ok, ok, 1024, 512, 99, None) == 2

@@ -286,3 +286,35 @@ print("OK")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "OK" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
+@pytest.mark.parametrize("T,E,k,dtype", [(4096, 8, 2, torch.bfloat16), (300, 8, 2, torch.float32), (1000, 16, 4, torch.bfloat16),
+                                         (1, 8, 2, torch.bfloat16), (777, 64, 8, torch.float32), (50, 5, 2, torch.bfloat16),
+                                         (513, 3, 3, torch.float32)])
+def test_moe_route_matches_torch(agemm, T, E, k, dtype):
+    """Softmax / top-k / normalised weights and the expert-sorted bookkeeping against torch's own operators
+    (model/qMixtralLayer.py:441-452 and what its loop over experts derives).  bf16 logits tie often; the library
+    takes the lower expert number among equals, which a stable descending sort reproduces."""
+    import torch.nn.functional as Fn
+    g = torch.Generator().manual_seed(T + E)
+    logits = (torch.randn(T, E, generator=g) * 2.0).to(dtype).cuda()
+    sel, w, seg, position, tok, ws = agemm.moe_route(logits, k)
+    p = Fn.softmax(logits, dim=1, dtype=torch.float)
+    vals, idx = torch.sort(p, dim=1, descending=True, stable=True)
+    want_sel, want_v = idx[:, :k], vals[:, :k]
+    assert torch.equal(sel.long(), want_sel)
+    want_w = (want_v / want_v.sum(dim=-1, keepdim=True)).to(torch.bfloat16)
+    if k == 2:
+        assert torch.equal(w, want_w)                      # same arithmetic as torch: same bits
+    else:                                                  # torch's sum over k > 2 values has its own order
+        assert float((w.float() - want_w.float()).abs().max()) <= 2.0 ** -8
+    flat = sel.long().reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    assert torch.equal(tok.long(), order // k)
+    assert torch.equal(ws, w.reshape(-1)[order])
+    want_seg = torch.zeros(E + 1, dtype=torch.int64, device="cuda")
+    want_seg[1:] = torch.cumsum(torch.bincount(flat, minlength=E), 0)
+    assert torch.equal(seg.long(), want_seg)
+    want_pos = torch.empty_like(order)
+    want_pos[order] = torch.arange(order.numel(), device="cuda")
+    assert torch.equal(position, want_pos)
