@@ -216,7 +216,8 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_place_kernel(int T, i
 
 extern "C" size_t arcq_moe_route_workspace_bytes(int tokens, int experts) {
   if (tokens < 0 || experts < 1) return 0;
-  return (size_t)((tokens + arcq::kRouteThreads - 1) / arcq::kRouteThreads) * (size_t)experts * sizeof(int);
+  const int blocks = tokens == 0 ? 1 : (tokens + arcq::kRouteThreads - 1) / arcq::kRouteThreads;
+  return (size_t)blocks * (size_t)experts * sizeof(int);
 }
 
 extern "C" int arcq_moe_route(const void *logits, int logits_f32, int tokens, int experts, int top_k, int *sel, void *weight,
@@ -227,7 +228,8 @@ extern "C" int arcq_moe_route(const void *logits, int logits_f32, int tokens, in
     return ARCQ_ERR_SHAPE;
   if (!seg_offsets) return ARCQ_ERR_NULL;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (!logits || !sel || !weight || !position || !token_of_row || !weight_of_row || !workspace) return ARCQ_ERR_NULL;
+  if (!workspace) return ARCQ_ERR_NULL;
+  if (tokens > 0 && (!logits || !sel || !weight || !position || !token_of_row || !weight_of_row)) return ARCQ_ERR_NULL;
   const int blocks = tokens == 0 ? 1 : (tokens + kRouteThreads - 1) / kRouteThreads;
   if (workspace_bytes < (size_t)blocks * experts * sizeof(int)) return ARCQ_ERR_WORKSPACE;
   int *hist = static_cast<int *>(workspace);

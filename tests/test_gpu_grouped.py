@@ -318,3 +318,9 @@ def test_moe_route_matches_torch(agemm, T, E, k, dtype):
     want_pos = torch.empty_like(order)
     want_pos[order] = torch.arange(order.numel(), device="cuda")
     assert torch.equal(position, want_pos)
+
+
+def test_moe_route_without_tokens(agemm):
+    sel, w, seg, position, tok, ws = agemm.moe_route(torch.empty((0, 8), dtype=torch.bfloat16, device="cuda"), 2)
+    assert sel.shape == (0, 2) and position.numel() == 0 and tok.numel() == 0
+    assert torch.equal(seg.cpu(), torch.zeros(9, dtype=torch.int32))
