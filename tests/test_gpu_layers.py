@@ -236,6 +236,44 @@ def test_mixtral_block_grouped_equals_loop_at_benchmark_size(layers):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
+def test_mixtral_block_replays_from_a_graph(layers, fmt):
+    """The grouped block reads nothing back to the host, so it can be captured: every replay (new tokens and
+    router logits copied into the captured inputs, eager work and a synchronisation between replays) gives
+    what the eager call gives on the same inputs."""
+    hidden, ffn, E, S, tokens = 384, 512, 4, 128, 96
+    g = torch.Generator().manual_seed(19)
+    block = layers.build_mixtral_block(hidden, ffn, E, 2, S, fmt, seed=7, grouped=True)
+    x_in = torch.zeros(1, tokens, hidden, dtype=torch.bfloat16, device="cuda")
+    l_in = torch.zeros(tokens, E, dtype=torch.float32, device="cuda")
+
+    def fresh():
+        return (torch.randn(1, tokens, hidden, generator=g).to(torch.bfloat16).cuda(),
+                torch.randn(tokens, E, generator=g).cuda())
+
+    x0, l0 = fresh()
+    x_in.copy_(x0), l_in.copy_(l0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                      # warm-up on the capture stream: allocations happen here
+        for _ in range(2):
+            block(x_in, router_logits=l_in)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    print(f"mixtral block graph capture {fmt}", flush=True)
+    with torch.cuda.graph(graph):
+        y_out, _ = block(x_in, router_logits=l_in)
+    for rep in range(3):
+        x1, l1 = fresh()
+        want, _ = block(x1, router_logits=l1)          # eager, between the replays
+        torch.cuda.synchronize()
+        x_in.copy_(x1), l_in.copy_(l1)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_out, want), rep
+
+
+@pytest.mark.parametrize("fmt", FMTS)
 def test_graphed_decode_step_matches_eager(layers, fmt):
     """A decode step over the INT4 paged KV cache replayed from a captured HIP graph gives what the
     eager step gives, on every replay, with eager work and synchronisation between replays, across a
