@@ -178,3 +178,26 @@ def test_matmul_with_residual_equals_separate_add(agemm, fmt, M, N, K, S):
     assert torch.equal(z, y + r)
     with pytest.raises(RuntimeError):
         agemm.matmul(a, b, sfa, sfb, gx * gw, residual=r[:, :-1].contiguous())
+
+
+def test_matmul_operand_of_more_than_4_gib(agemm):
+    """An activation operand of 4.35 GB (2 000 000 rows of K' = 4352): the eight-wave MXFP4 kernels address rows
+    with 32-bit byte offsets, so the dispatch must hand this one to the kernels with 64-bit addresses.  Random
+    codes and scale bytes near 2^0; first, middle and last rows against the product of the dequantized operands."""
+    M, N, Kp = 2_000_000, 512, 4352
+    g = torch.Generator(device="cuda").manual_seed(1)
+    a = torch.randint(0, 256, (M, Kp // 2), dtype=torch.uint8, device="cuda", generator=g)
+    b = torch.randint(0, 256, (N, Kp // 2), dtype=torch.uint8, device="cuda", generator=g)
+    sfa = torch.randint(124, 130, (M * (Kp // 32),), dtype=torch.uint8, device="cuda", generator=g)
+    sfb = torch.randint(124, 130, (N * (Kp // 32),), dtype=torch.uint8, device="cuda", generator=g)
+    assert a.numel() >= 1 << 32
+    print(f"matmul MXFP4 M={M} N={N} K'={Kp}: operand of {a.numel()} bytes", flush=True)
+    c = agemm.matmul(a, b, sfa, sfb, 1.0, fmt="MXFP4")
+    db = agemm.dequantize(b, sfb, fmt="MXFP4")
+    for r0 in (0, M // 2 + 3, 1_999_000, M - 64):
+        da = agemm.dequantize(a[r0:r0 + 64].contiguous(), sfa.view(M, -1)[r0:r0 + 64].contiguous().view(-1), fmt="MXFP4")
+        want = da @ db.T
+        err = float((c[r0:r0 + 64].float() - want).norm() / want.norm())
+        assert err < 5e-3, (r0, err)
+    del a, c
+    torch.cuda.empty_cache()
