@@ -790,7 +790,8 @@ __global__ __launch_bounds__(128 * NWM) void gemm_nvfp4_tiled(GemmParams p) {
   constexpr int BN = 64 * WN, BM = 32 * WM * NWM, NW = 2 * NWM;
   constexpr int RPI = 16 * NWM;  // rows of 128 code bytes that one load instruction of the workgroup covers
   __shared__ uint4 sW[2 * BN * 8], sX[2 * BM * 8];  // code tiles, two stages each
-  __shared__ uint4 sWs[2 * BN], sXs[2 * BM];        // 16 scale bytes per row per K step, two stages each
+  constexpr int BMS = BM < 64 ? 64 : BM;            // a scale load instruction covers 64 rows (clamped to the last one)
+  __shared__ uint4 sWs[2 * BN], sXs[2 * BMS];       // 16 scale bytes per row per K step, two stages each
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kbytes = p.Kp >> 1, ksc = p.Kp >> 4;
@@ -822,11 +823,11 @@ __global__ __launch_bounds__(128 * NWM) void gemm_nvfp4_tiled(GemmParams p) {
   // scales: one lane = the 16 scale bytes of one row for this K step; instruction j (64 rows) of
   // the weights goes to wave j%4, of the activations to wave (j+WN)%4.  In a short last step the
   // window is shifted back by 8 bytes so that it ends with the row.
-  const uint8_t *wssrc[BN / 64], *xssrc[BM / 64];
+  const uint8_t *wssrc[BN / 64], *xssrc[BMS / 64];
 #pragma unroll
   for (int j = 0; j < BN / 64; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
 #pragma unroll
-  for (int j = 0; j < BM / 64; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
+  for (int j = 0; j < BMS / 64; ++j) xssrc[j] = p.a_scales + (size_t)min(m_base + 64 * j + lane, p.M - 1) * ksc;
   const uint32_t lw0 = (uint32_t)reinterpret_cast<uintptr_t>(sW) + wave * 1024;
   const uint32_t lx0 = (uint32_t)reinterpret_cast<uintptr_t>(sX) + wave * 1024;
   const uint32_t lws0 = (uint32_t)reinterpret_cast<uintptr_t>(sWs);
@@ -845,8 +846,8 @@ __global__ __launch_bounds__(128 * NWM) void gemm_nvfp4_tiled(GemmParams p) {
     for (int j = 0; j < BN / 64; ++j)
       if ((j % NW) == wave) lds_dma16(wssrc[j] + soff, lws0 + st * (BN * 16) + j * 1024);
 #pragma unroll
-    for (int j = 0; j < BM / 64; ++j)
-      if (((j + BN / 64) % NW) == wave) lds_dma16(xssrc[j] + soff, lxs0 + st * (BM * 16) + j * 1024);
+    for (int j = 0; j < BMS / 64; ++j)
+      if (((j + BN / 64) % NW) == wave) lds_dma16(xssrc[j] + soff, lxs0 + st * (BMS * 16) + j * 1024);
   };
 
   const int r = lane & 31, kh = lane >> 5;
@@ -891,7 +892,7 @@ __global__ __launch_bounds__(128 * NWM) void gemm_nvfp4_tiled(GemmParams p) {
     }
 #pragma unroll
     for (int j = 0; j < WM; ++j) {
-      const uint2 b = reinterpret_cast<const uint2 *>(sXs + st * BM + wm0 + r + 32 * j)[sq];
+      const uint2 b = reinterpret_cast<const uint2 *>(sXs + st * BMS + wm0 + r + 32 * j)[sq];
       xsp[j][0] = nv_scale_pair_f16(b.x & 0x00ff00ffu);
       xsp[j][1] = nv_scale_pair_f16((b.x >> 8) & 0x00ff00ffu);
       xsp[j][2] = nv_scale_pair_f16(b.y & 0x00ff00ffu);
@@ -1242,7 +1243,13 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
   // so it pays only where the single launch is far from the weight stream's time).
   int split = 0;
   bool one_round_21 = false;  // 128x64 tiles, no more of them than CUs, K not cut
+  // NVFP4 on a wide layer with up to 32 rows: decoding bounds the 128x64 tile (every weight row decoded by both
+  // of its M-waves, 64 activation rows multiplied of which at most 32 are real), so workgroups of two waves along
+  // N with a 64x32 tile -- each weight row decoded once -- and K in two slices to fill the CUs
+  // (gate_up 28672 x 4096: 30.7 -> 24.7 us at M = 16, 28.7 -> 26.7 at M = 32; slower on the narrow layers)
+  const bool small_nv = fmt == ARCQ_FMT_NVFP4 && split_env == 0 && force < 0 && M >= 8 && M <= 32 && N >= 16384 && Kp < 8192;
   if (split_env > 1) split = M <= 512 ? split_env : 0;
+  else if (small_nv) split = 2;
   else if (split_env == 0 && force < 0 && M <= 64 && N <= 8192) {
     if (Kp >= 8192 && M >= 24) split = 8;
     else if (Kp < 8192 && N > 4096 && M > (fmt == ARCQ_FMT_MXFP4 ? 16 : 32)) split = 4;
@@ -1264,7 +1271,7 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
     const int slices = std::min(split, (Kp + 255) / 256 / 2);
     const size_t bytes = (size_t)slices * M * N * sizeof(float);
     if (slices > 1 && bytes <= kSplitMaxBytes) {
-      plan.kernel = fmt == ARCQ_FMT_MXFP4 ? 214 : 21;
+      plan.kernel = fmt == ARCQ_FMT_MXFP4 ? 214 : ((small_nv || force == 11) ? 11 : 21);
       plan.slices = slices;
       plan.scratch = bytes;
       return plan;
@@ -1309,7 +1316,7 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
     // against 74 us with 256x128 tiles), so the next smaller tile that still fills it
     const long t44 = (long)((M + 255) / 256) * ((N + 255) / 256), t42 = (long)((M + 127) / 128) * ((N + 255) / 256);
     const int pick = t44 >= 192 ? 44 : (M > 128 && !one_round_21 ? (t42 >= 192 ? 42 : 22) : 21);
-    const bool known = force == 44 || force == 84 || force == 42 || force == 22 || force == 21;
+    const bool known = force == 44 || force == 84 || force == 42 || force == 22 || force == 21 || force == 11;
     plan.kernel = known ? force : pick;  // a forced kernel that NVFP4 does not have is ignored
     return plan;
   }
@@ -1321,7 +1328,8 @@ int run_gemm(GemmParams p, const GemmPlan &plan, int fmt, float *scratch, hipStr
   if (plan.slices > 1) {
     p.k_slices = plan.slices;
     p.partial = scratch;
-    const int rc = fmt == ARCQ_FMT_MXFP4 ? launch_mxfp4_tiled<2, 1, 4>(p, st) : launch_nvfp4_tiled<2, 1>(p, st);
+    const int rc = fmt == ARCQ_FMT_MXFP4 ? launch_mxfp4_tiled<2, 1, 4>(p, st)
+                   : (plan.kernel == 11 ? launch_nvfp4_tiled<1, 1, 1>(p, st) : launch_nvfp4_tiled<2, 1>(p, st));
     if (rc != ARCQ_OK) return rc;
     const size_t total4 = ((size_t)p.M * p.N) >> 2;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<size_t>((total4 + 255) / 256, 1024)), dim3(256), 0,
@@ -1352,6 +1360,7 @@ int run_gemm(GemmParams p, const GemmPlan &plan, int fmt, float *scratch, hipStr
       case 42: return launch_nvfp4_tiled<4, 2>(p, st);
       case 22: return launch_nvfp4_tiled<2, 2>(p, st);
       case 21: return launch_nvfp4_tiled<2, 1>(p, st);
+      case 11: return launch_nvfp4_tiled<1, 1, 1>(p, st);  // 64x32 tile, two waves along N
       default: break;
     }
   }

@@ -38,7 +38,7 @@ constexpr size_t kWorkspaceBytes[kWsKinds] = {256, 32u << 20, 8u << 20};
 void *stream_workspace(int kind, hipStream_t stream, int *status);
 
 // Overrides for tuning runs, read from the environment once, when the library is first used:
-//   ARCQ_GEMM_KERNEL=<WN><WM>   force a GEMM tile (84 / 82 = 256x256 / 256x128 as eight waves, 44, 42, 22, 21; 214 / 224 = four-stage
+//   ARCQ_GEMM_KERNEL=<WN><WM>   force a GEMM tile (84 / 82 = 256x256 / 256x128 as eight waves, 44, 42, 22, 21, 11; 214 / 224 = four-stage
 //                               ring; 1 = skinny, 0 = direct); a number the format has no kernel for is ignored
 //   ARCQ_GEMM_SPLITK=<slices>   force split-K for M <= 512 (1 = never split)
 //   ARCQ_QUANT_GRID=<n>         workgroups of the row quantizers

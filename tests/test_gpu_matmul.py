@@ -125,7 +125,7 @@ def test_matmul_llama_shapes_vs_torch_fp32(agemm, oracle, fmt, M, N, K, S):
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 32, 48, 64])
 @pytest.mark.parametrize("N,K,S", [(6144, 4096, 256), (202, 384, 0), (4100, 1024, 128), (4100, 8192, 128),
-                                   (8324, 1024, 256), (8450, 768, 256)])
+                                   (8324, 1024, 256), (8450, 768, 256), (16500, 1024, 128)])
 def test_matmul_decode_batches(agemm, oracle, fmt, M, N, K, S):
     """M <= 64 (decode batches) at a benchmark shape and at shapes whose N is not a multiple of the
     16-row strips or of the 4-wide stores: against torch's fp32 matmul of the dequantized operands,
