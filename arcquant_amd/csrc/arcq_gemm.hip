@@ -1247,7 +1247,10 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
   // of its M-waves, 64 activation rows multiplied of which at most 32 are real), so workgroups of two waves along
   // N with a 64x32 tile -- each weight row decoded once -- and K in two slices to fill the CUs
   // (gate_up 28672 x 4096: 30.7 -> 24.7 us at M = 16, 28.7 -> 26.7 at M = 32; slower on the narrow layers)
-  const bool small_nv = fmt == ARCQ_FMT_NVFP4 && split_env == 0 && force < 0 && M >= 8 && M <= 32 && N >= 16384 && Kp < 8192;
+  // (only while the two slices fit the 8 MiB array of the entry point that allocates nothing, which serves
+  // every decode batch: N up to 32768 at 32 rows)
+  const bool small_nv = fmt == ARCQ_FMT_NVFP4 && split_env == 0 && force < 0 && M >= 8 && M <= 32 && N >= 16384 && Kp < 8192 &&
+                        (size_t)2 * M * N * sizeof(float) <= ((size_t)8 << 20);
   if (split_env > 1) split = M <= 512 ? split_env : 0;
   else if (small_nv) split = 2;
   else if (split_env == 0 && force < 0 && M <= 64 && N <= 8192) {
