@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t *y, con
 // Equal probabilities: the lower expert number wins (torch.topk leaves the choice among equals unspecified).
 // ---------------------------------------------------------------------------------------------
 constexpr int kMaxExperts = 64;
-constexpr int kRouteThreads = 256;
+constexpr int kRouteThreads = 64;
 
 template <bool F32, int P>  // P: the power of two the experts are padded to
 __global__ __launch_bounds__(kRouteThreads) void moe_route_choose_kernel(const void *logits, int T, int E, int top_k, int *sel,

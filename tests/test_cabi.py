@@ -103,7 +103,7 @@ def test_grouped_entry_points_reject_bad_arguments():
     assert mc(ok, None, ok, 8, 4096, 2, 16, ok, None) == 1
     assert mc(ok, ok, ok, 0, 4096, 2, 0, ok, None) == 0
     mr = L.arcq_moe_route
-    assert L.arcq_moe_route_workspace_bytes(4096, 8) == 16 * 8 * 4
+    assert L.arcq_moe_route_workspace_bytes(4096, 8) == 64 * 8 * 4
     assert mr(ok, 0, 16, 65, 2, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None) == 2               # more than 64 experts
     assert mr(ok, 0, 16, 8, 9, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None) == 2                # top_k > 8
     assert mr(ok, 0, 16, 4, 5, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None) == 2                # top_k > experts
