@@ -182,22 +182,37 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_place_kernel(int T, i
                                                                         const int *hist, int64_t *position, int *seg, int *tok,
                                                                         uint16_t *ws) {
   __shared__ int start[kMaxExperts];  // first sorted row of this workgroup's pairs of expert e
-  if (threadIdx.x < E) {
-    const int e = threadIdx.x;
-    int before = 0;  // pairs of experts below e, plus those of e in earlier workgroups
-    for (int b = 0; b < (int)gridDim.x; ++b)
-      for (int q = 0; q < e; ++q) before += hist[(size_t)b * E + q];
-    int seg_e = before;
-    for (int b = 0; b < (int)blockIdx.x; ++b) before += hist[(size_t)b * E + e];
-    start[e] = before;
-    if (blockIdx.x == 0) {
-      seg[e] = seg_e;
-      if (e == E - 1) {
-        int all = seg_e;
-        for (int b = 0; b < (int)gridDim.x; ++b) all += hist[(size_t)b * E + e];
-        seg[E] = all;
+  __shared__ int total[kMaxExperts], earlier[kMaxExperts];
+  if (threadIdx.x < kMaxExperts) total[threadIdx.x] = earlier[threadIdx.x] = 0;
+  __syncthreads();
+  // The histograms [workgroups][E] were written on other XCDs and come from memory: a lane takes eight of
+  // their words at a time, all eight loads in flight together, and adds them to the experts' sums in LDS.
+  const int words = (int)gridDim.x * E, mine = (int)blockIdx.x * E;  // words below `mine` belong to earlier workgroups
+  for (int f0 = 0; f0 < words; f0 += 8 * kRouteThreads) {
+    int v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int fl = f0 + u * kRouteThreads + (int)threadIdx.x;
+      v[u] = fl < words ? hist[fl] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int fl = f0 + u * kRouteThreads + (int)threadIdx.x;
+      if (fl < words && v[u]) {
+        atomicAdd(&total[fl % E], v[u]);
+        if (fl < mine) atomicAdd(&earlier[fl % E], v[u]);
       }
     }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = run + earlier[e];
+      if (blockIdx.x == 0) seg[e] = run;
+      run += total[e];
+    }
+    if (blockIdx.x == 0) seg[E] = run;
   }
   __syncthreads();
   const int t = blockIdx.x * kRouteThreads + threadIdx.x;
