@@ -939,8 +939,10 @@ __global__ __launch_bounds__(256) void tensor_scale_kernel(const uint16_t *x, co
 
 // Per-segment maxima for grouped launches (rows sorted by segment): max |x|, or max |act_fn(gate) * up|,
 // over the rows of each segment, accumulated as the bits of a non-negative float in bits[segment] (zeroed
-// by the caller's launch in front).  A workgroup walks rows with stride gridDim and flushes its running
-// maximum with one atomicMax when its rows enter another segment, and at the end.
+// by the caller's launch in front).  A workgroup takes a contiguous run of rows and flushes its running
+// maximum with one atomicMax when its rows enter another segment, and at the end: atomics on one word are
+// served one after the other (about 10 ns each), so there must be few of them -- with rows dealt out
+// round-robin every row of every workgroup ended in one (8192 rows over 8 segments: 86 us, all of it waiting).
 template <bool SWIGLU>
 __global__ __launch_bounds__(256) void grouped_absmax_kernel(const uint16_t *x, const uint16_t *up, size_t ld, int rows,
                                                              int K, const int *seg, int n_seg, uint32_t *bits) {
@@ -964,7 +966,9 @@ __global__ __launch_bounds__(256) void grouped_absmax_kernel(const uint16_t *x, 
     }
     m = 0u;
   };
-  for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+  const int per_wg = (rows + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int r_end = min(rows, ((int)blockIdx.x + 1) * per_wg);
+  for (int r = (int)blockIdx.x * per_wg; r < r_end; ++r) {
     if (r >= seg_end) {
       flush();
       while (seg_cur + 1 < n_seg && r >= seg_end) {
@@ -978,12 +982,12 @@ __global__ __launch_bounds__(256) void grouped_absmax_kernel(const uint16_t *x, 
     }
     // four rows of the workgroup at a time while they stay inside the segment: all their loads are issued
     // before the first maximum is taken (a row of a few thousand channels is only two loads per thread)
-    const int nr = (!SWIGLU && (long)r + 3L * gridDim.x < (long)min(seg_end, rows)) ? 4 : 1;
+    const int nr = (!SWIGLU && r + 3 < min(seg_end, r_end)) ? 4 : 1;
     for (int c = threadIdx.x; c < cpr; c += 256) {
       uint4 gq[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        if (j < nr) gq[j] = *reinterpret_cast<const uint4 *>(x + (size_t)(r + j * (int)gridDim.x) * ld + 8 * c);
+        if (j < nr) gq[j] = *reinterpret_cast<const uint4 *>(x + (size_t)(r + j) * ld + 8 * c);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (j >= nr) break;
@@ -1001,7 +1005,7 @@ __global__ __launch_bounds__(256) void grouped_absmax_kernel(const uint16_t *x, 
         }
       }
     }
-    r += (nr - 1) * (int)gridDim.x;
+    r += nr - 1;
   }
   flush();
 }
@@ -1450,7 +1454,7 @@ int arcq_grouped_tensor_scale(const void *x, const void *up, int ld, int M, int 
   const int fin = (n_seg + 255) / 256;
   hipLaunchKernelGGL(arcq::zero_words_kernel, dim3(fin), dim3(256), 0, st, bits, n_seg);
   if (M > 0) {
-    const int grid = M < 2048 ? M : 2048;
+    const int grid = std::min(1024, (M + 7) / 8);  // eight or more contiguous rows per workgroup
     if (up)
       hipLaunchKernelGGL(arcq::grouped_absmax_kernel<true>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(x),
                          static_cast<const uint16_t *>(up), (size_t)ld, M, K, seg_offsets, n_seg, bits);
