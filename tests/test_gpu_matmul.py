@@ -201,3 +201,34 @@ def test_matmul_operand_of_more_than_4_gib(agemm):
         assert err < 5e-3, (r0, err)
     del a, c
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("seed", [1, 7])
+def test_matmul_random_shapes(agemm, seed):
+    """Forty random (format, M, N, K, select_num) problems per seed, sizes around the tile edges of every
+    kernel the dispatch knows: quantize both operands, multiply, compare with the product of the dequantized
+    operands (the rounding of the bf16 output bounds the error)."""
+    import random
+    rnd = random.Random(seed)
+    done = 0
+    while done < 40:
+        fmt = rnd.choice(FMTS)
+        M = rnd.choice([1, 2, 7, 16, 17, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 200, 255, 256, 257, 300, 511, 512, 513, 700,
+                        1000, 1024, 1500, 2048, 2100, 3000])
+        N = rnd.choice([8, 16, 24, 64, 100, 128, 136, 200, 256, 264, 500, 512, 520, 1000, 1024, 2048, 2056, 4096, 4104, 6144,
+                        8192, 8200, 16384, 28672])
+        K = rnd.choice([64, 128, 192, 256, 320, 384, 448, 512, 640, 768, 896, 1024, 1152, 2048, 3072, 4096])
+        S = min(rnd.choice([0, 64, 128, 256]), K)
+        if M * N > 12_000_000 or N * K > 60_000_000:
+            continue
+        x = recipes.activations(M, K, seed=seed * 1000 + done, outlier_frac=0.01, outlier_gain=30.0).cuda()
+        w = recipes.weights(N, K, seed=seed * 2000 + done).cuda()
+        idx = torch.randperm(K, generator=torch.Generator().manual_seed(done)).to(torch.int16).cuda()
+        print(f"random shape {done}: {fmt} M={M} N={N} K={K} S={S}", flush=True)
+        a, sfa = agemm.reorder_quantize_x(x, idx, S, fmt=fmt)
+        b, sfb = agemm.reorder_quantize_w(w, idx, S, fmt=fmt)
+        y = agemm.matmul(a, b, sfa, sfb, 1.0, fmt=fmt)
+        want = agemm.dequantize(a, sfa, fmt=fmt) @ agemm.dequantize(b, sfb, fmt=fmt).T
+        err = float((y.float() - want).norm() / max(1e-20, float(want.norm())))
+        assert err < 6e-3, (fmt, M, N, K, S, err)
+        done += 1
