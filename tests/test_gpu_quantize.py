@@ -248,3 +248,37 @@ def test_tensor_scale_matches_torch(agemm, M, K):
         assert float(got) == float(want)
     assert float(agemm.tensor_scale(torch.zeros(M, K, dtype=torch.bfloat16, device="cuda"))) == 1.0
     assert float(agemm.tensor_scale(view.contiguous(), 6.0)) == float(view.abs().max().float() / torch.full((), 6.0, device="cuda"))
+
+
+@pytest.mark.parametrize("seed", [3, 11])
+def test_quantizers_random_shapes(agemm, oracle, seed):
+    """Thirty random (operator, format, rows, K, select_num, tensor scale) problems per seed around the row
+    counts and widths where the dispatch changes kernels: codes and scale bytes bit for bit against the oracle."""
+    import random
+    rnd = random.Random(seed)
+    done = 0
+    while done < 30:
+        fmt = rnd.choice(FMTS)
+        G = 16 if fmt == "NVFP4" else 32
+        mode = rnd.choice(["x", "w", "norm", "norm", "x"])
+        M = rnd.choice([1, 2, 3, 15, 16, 17, 64, 100, 255, 256, 257, 1000, 3071, 3072, 3073, 4096, 5000])
+        K = rnd.choice([32, 64, 96, 128, 512, 1024, 2048, 3072, 3584, 4096, 5120, 8192, 14336])
+        S = min(rnd.choice([0, G, 64, 128, 256, 512]), K)
+        if M * K > 13_000_000:
+            continue
+        x = recipes.activations(M, K, seed=seed * 100 + done, outlier_frac=0.01, outlier_gain=50.0)
+        idx = recipes.reorder_index(x)
+        gs = rnd.choice([1.0, recipes.tensor_scale(x, fmt)])
+        print(f"random quantizer {done}: {mode} {fmt} M={M} K={K} S={S} gscale={gs}", flush=True)
+        if mode == "x":
+            want = oracle.quantize_x(x, idx, S, fmt, gs)
+            q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), S, fmt=fmt, global_scale=gs)
+        elif mode == "w":
+            want = oracle.quantize_w(x, idx, S, fmt, gs)
+            q, sf = agemm.reorder_quantize_w(dev(x), dev(idx), S, fmt=fmt, global_scale=gs)
+        else:
+            gamma = (1.0 + 0.1 * torch.randn(K, generator=torch.Generator().manual_seed(done))).to(torch.bfloat16)
+            want = oracle.rmsnorm_quantize_x(x, gamma, 1e-5, idx, S, fmt, gs)
+            q, sf = agemm.rmsnorm_quantize_x(dev(x), dev(gamma), 1e-5, dev(idx), S, fmt=fmt, global_scale=gs)
+        compare(f"{mode} {fmt} M={M} K={K} S={S}", q, sf, want)
+        done += 1
