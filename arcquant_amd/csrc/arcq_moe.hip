@@ -81,6 +81,10 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t *y, con
 // exp(l - max) as the butterfly over the next power of two that its warp softmax forms (padding adds zeros),
 // exp(l - max) / sum, top-k weights divided by their sum left to right (exact for k = 2, the Mixtral case).
 // Equal probabilities: the lower expert number wins (torch.topk leaves the choice among equals unspecified).
+// Non-finite logits (a NaN, a +inf, or a row of -inf) make every probability of the row NaN, as in torch; the
+// choice stays total -- NaN ranks above every number, as torch.topk orders it, and equals again go to the lower
+// expert -- so every pair names an expert in [0, E), is counted in the histograms and gets a row; only that
+// token's weights, and through them its output, are NaN.
 // ---------------------------------------------------------------------------------------------
 constexpr int kMaxExperts = 64;
 constexpr int kRouteThreads = 64;
@@ -137,7 +141,8 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_choose_kernel(const v
         bool taken = false;
 #pragma unroll
         for (int q = 0; q < kMaxTopK; ++q) taken |= q < j && my[q] == e;
-        if (e < E && !taken && prob[e] > bv) { bv = prob[e]; best = e; }
+        const bool above = prob[e] != prob[e] ? bv == bv : prob[e] > bv;  // NaN above every number, not above NaN
+        if (e < E && !taken && (best < 0 || above)) { bv = prob[e]; best = e; }
       }
       my[j] = best;
       mw[j] = bv;
@@ -219,6 +224,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_place_kernel(int T, i
   if (t >= T) return;
   for (int j = 0; j < top_k; ++j) {
     const size_t pair = (size_t)t * top_k + j;
+    if ((unsigned)sel[pair] >= (unsigned)E) continue;  // cannot happen with the choice above; never index LDS with it
     const int64_t pos = start[sel[pair]] + position[pair];
     position[pair] = pos;
     tok[pos] = t;

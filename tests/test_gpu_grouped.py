@@ -324,3 +324,62 @@ def test_moe_route_without_tokens(agemm):
     sel, w, seg, position, tok, ws = agemm.moe_route(torch.empty((0, 8), dtype=torch.bfloat16, device="cuda"), 2)
     assert sel.shape == (0, 2) and position.numel() == 0 and tok.numel() == 0
     assert torch.equal(seg.cpu(), torch.zeros(9, dtype=torch.int32))
+
+
+def test_moe_route_with_non_finite_logits(agemm):
+    """A NaN logit, a +inf logit or a row of -inf makes every probability of that row NaN (torch's softmax
+    does the same).  The routing must stay a routing: every choice an expert number, every pair counted in the
+    segments and given a row of its own, and only the affected tokens' weights NaN."""
+    T, E, k = 200, 8, 2
+    g = torch.Generator().manual_seed(12)
+    logits = (torch.randn(T, E, generator=g) * 2.0).to(torch.bfloat16)
+    bad = [3, 64, 65, 199]
+    logits[3, 5] = float("nan")
+    logits[64, 0] = float("inf")
+    logits[65] = float("-inf")
+    logits[199, 7] = float("nan")
+    logits[199, 1] = float("inf")
+    sel, w, seg, position, tok, ws = agemm.moe_route(logits.cuda(), k)
+    torch.cuda.synchronize()
+    sel, w, seg, position, tok = sel.cpu(), w.cpu(), seg.cpu(), position.cpu(), tok.cpu()
+    assert int(sel.min()) >= 0 and int(sel.max()) < E
+    assert all(len(set(r.tolist())) == k for r in sel)                 # a token never takes an expert twice
+    assert int(seg[E]) == T * k and int(seg[0]) == 0
+    assert torch.equal(seg[1:] - seg[:-1], torch.bincount(sel.reshape(-1).long(), minlength=E).int())
+    assert torch.equal(torch.sort(position).values, torch.arange(T * k))          # a permutation of the pairs
+    assert torch.equal(tok.long(), torch.argsort(sel.reshape(-1).long(), stable=True) // k)
+    nan_rows = torch.isnan(w.float()).any(1).nonzero().flatten().tolist()
+    assert nan_rows == bad
+    # NaN ranks above every number and equals go to the lower expert: all-NaN rows take experts 0 and 1
+    assert all(sel[t].tolist() == [0, 1] for t in bad)
+    # the other tokens are routed as torch routes them
+    import torch.nn.functional as Fn
+    ok = torch.tensor([t for t in range(T) if t not in bad])
+    p = Fn.softmax(logits[ok].float(), dim=1)
+    vals, order = torch.sort(p, dim=1, descending=True, stable=True)
+    assert torch.equal(sel[ok].long(), order[:, :k])
+
+
+def test_mixtral_block_with_non_finite_logits():
+    """the whole block on such logits: finite outputs for every token but the affected ones"""
+    from arcquant_amd import layers
+    hidden, ffn, E = 512, 1024, 8
+    blk = layers.build_mixtral_block(hidden=hidden, ffn=ffn, num_experts=E, select_num=128, quant_type="NVFP4", seed=3)
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(1, 96, hidden, generator=g).to(torch.bfloat16).cuda()
+    logits = (torch.randn(96, E, generator=g) * 2.0).to(torch.bfloat16)
+    logits[7, 2] = float("nan")
+    logits[40] = float("-inf")
+    logits[95, 3] = float("inf")
+    y, _ = blk(x, router_logits=logits.cuda())
+    torch.cuda.synchronize()
+    nan_tokens = torch.isnan(y[0].float()).any(1).nonzero().flatten().tolist()
+    assert nan_tokens == [7, 40, 95]
+    clean = torch.tensor([t for t in range(96) if t not in (7, 40, 95)]).cuda()
+    logits2 = logits.clone()
+    logits2[[7, 40, 95]] = 0.0
+    y2, _ = blk(x, router_logits=logits2.cuda())
+    # NVFP4's per-expert tensor scales see the same activations either way unless an affected token is an expert's
+    # maximum; the clean tokens' outputs stay finite and close to the run without the bad logits
+    assert bool(torch.isfinite(y[0][clean].float()).all())
+    assert rel_fro(y[0][clean].float(), y2[0][clean].float()) < 5e-2

@@ -159,7 +159,7 @@ def test_llama_mlp_fused_swiglu_equals_separate_pass(layers, fmt, tokens):
 
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("grouped,interleave", [(True, True), (True, False), (False, True), (False, False)])
-def test_mixtral_block_matches_reference_loop(layers, fq, fmt, grouped, interleave):
+def test_mixtral_block_matches_reference_loop(layers, fq, oracle, fmt, grouped, interleave):
     """The MoE block, as grouped launches over all experts and as the per-expert loop, against the
     reference's loop (model/qMixtralLayer.py:441-471) on the CPU; every expert has its own channel orders."""
     hidden, ffn, E, S = 384, 512, 4, 128
@@ -177,8 +177,11 @@ def test_mixtral_block_matches_reference_loop(layers, fq, fmt, grouped, interlea
     y, _ = block(x.cuda(), router_logits=logits.cuda())
     assert y.shape == x.shape
 
-    # model/qMixtralLayer.py:441-471 on the CPU; expert weights = dequantised w13 / w2 of the block
-    from arcquant_amd import agemm
+    # model/qMixtralLayer.py:441-471 on the CPU; expert weights = w13 / w2 of the block as the CPU oracle dequantizes them
+    def dq(lin):
+        n = lin.W.shape[0]
+        v = oracle.dequantize(lin.W.cpu().numpy(), lin.scale_w.cpu().numpy().reshape(n, -1), fmt)
+        return torch.from_numpy(v) * lin.scale.cpu().float()
     w = F.softmax(logits, dim=1, dtype=torch.float)
     w, sel = torch.topk(w, 2, dim=-1)
     w = (w / w.sum(dim=-1, keepdim=True)).to(torch.bfloat16)
@@ -190,10 +193,10 @@ def test_mixtral_block_matches_reference_loop(layers, fq, fmt, grouped, interlea
             continue
         ex = block.experts[e]
         ih, ii = indices[e][0].cpu(), indices[e][1].cpu()
-        w13 = (agemm.dequantize(ex.w13.W.contiguous(), ex.w13.scale_w.contiguous(), fmt=fmt) * ex.w13.scale).cpu()
+        w13 = dq(ex.w13)
         if ex.interleaved:                                  # rows w1_0, w3_0, w1_1, ... -> [w1 | w3]
             w13 = torch.cat([w13[0::2], w13[1::2]])
-        w2 = (agemm.dequantize(ex.w2.W.contiguous(), ex.w2.scale_w.contiguous(), fmt=fmt) * ex.w2.scale).cpu()
+        w2 = dq(ex.w2)
         cur = x2[top_x]
         hcur = (ref_quant_x(fq, cur, ih, S, fmt) @ w13.T).to(torch.bfloat16)
         t = F.silu(hcur[:, :ffn]) * hcur[:, ffn:]

@@ -180,10 +180,17 @@ def test_matmul_with_residual_equals_separate_add(agemm, fmt, M, N, K, S):
         agemm.matmul(a, b, sfa, sfb, gx * gw, residual=r[:, :-1].contiguous())
 
 
-def test_matmul_operand_of_more_than_4_gib(agemm):
+def oracle_dq(oracle, q, sf, fmt):
+    """fp32 values of quantized rows from the CPU oracle's dequantizer, on the GPU"""
+    rows = q.shape[0]
+    return torch.from_numpy(oracle.dequantize(q.cpu().numpy(), sf.cpu().numpy().reshape(rows, -1), fmt)).cuda()
+
+
+def test_matmul_operand_of_more_than_4_gib(agemm, oracle):
     """An activation operand of 4.35 GB (2 000 000 rows of K' = 4352): the eight-wave MXFP4 kernels address rows
     with 32-bit byte offsets, so the dispatch must hand this one to the kernels with 64-bit addresses.  Random
-    codes and scale bytes near 2^0; first, middle and last rows against the product of the dequantized operands."""
+    codes and scale bytes near 2^0; first, middle and last rows against the product of the operands as the CPU
+    oracle dequantizes them."""
     M, N, Kp = 2_000_000, 512, 4352
     g = torch.Generator(device="cuda").manual_seed(1)
     a = torch.randint(0, 256, (M, Kp // 2), dtype=torch.uint8, device="cuda", generator=g)
@@ -193,21 +200,24 @@ def test_matmul_operand_of_more_than_4_gib(agemm):
     assert a.numel() >= 1 << 32
     print(f"matmul MXFP4 M={M} N={N} K'={Kp}: operand of {a.numel()} bytes", flush=True)
     c = agemm.matmul(a, b, sfa, sfb, 1.0, fmt="MXFP4")
-    db = agemm.dequantize(b, sfb, fmt="MXFP4")
+    db = oracle_dq(oracle, b, sfb, "MXFP4")
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
     for r0 in (0, M // 2 + 3, 1_999_000, M - 64):
-        da = agemm.dequantize(a[r0:r0 + 64].contiguous(), sfa.view(M, -1)[r0:r0 + 64].contiguous().view(-1), fmt="MXFP4")
+        da = oracle_dq(oracle, a[r0:r0 + 64], sfa.view(M, -1)[r0:r0 + 64], "MXFP4")
         want = da @ db.T
         err = float((c[r0:r0 + 64].float() - want).norm() / want.norm())
         assert err < 5e-3, (r0, err)
+    torch.backends.cuda.matmul.allow_tf32 = prev
     del a, c
     torch.cuda.empty_cache()
 
 
 @pytest.mark.parametrize("seed", [1, 7])
-def test_matmul_random_shapes(agemm, seed):
+def test_matmul_random_shapes(agemm, oracle, seed):
     """Forty random (format, M, N, K, select_num) problems per seed, sizes around the tile edges of every
-    kernel the dispatch knows: quantize both operands, multiply, compare with the product of the dequantized
-    operands (the rounding of the bf16 output bounds the error)."""
+    kernel the dispatch knows: quantize both operands, multiply, compare the whole output with the fp32 product
+    of the operands as the CPU oracle dequantizes them (the rounding of the bf16 output bounds the error)."""
     import random
     rnd = random.Random(seed)
     done = 0
@@ -228,7 +238,7 @@ def test_matmul_random_shapes(agemm, seed):
         a, sfa = agemm.reorder_quantize_x(x, idx, S, fmt=fmt)
         b, sfb = agemm.reorder_quantize_w(w, idx, S, fmt=fmt)
         y = agemm.matmul(a, b, sfa, sfb, 1.0, fmt=fmt)
-        want = agemm.dequantize(a, sfa, fmt=fmt) @ agemm.dequantize(b, sfb, fmt=fmt).T
+        want = oracle_dq(oracle, a, sfa, fmt) @ oracle_dq(oracle, b, sfb, fmt).T
         err = float((y.float() - want).norm() / max(1e-20, float(want.norm())))
         assert err < 6e-3, (fmt, M, N, K, S, err)
         done += 1

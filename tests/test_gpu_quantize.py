@@ -61,7 +61,8 @@ def test_reorder_quantize_w(agemm, oracle, fmt, N, K, S):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-@pytest.mark.parametrize("M,K,S", [(1, 4096, 64), (16, 4096, 256), (256, 4096, 64), (19, 8192, 256), (6, 2048, 0)])
+@pytest.mark.parametrize("M,K,S", [(1, 4096, 64), (1, 4096, 256), (16, 4096, 64), (16, 4096, 256), (256, 4096, 64),
+                                   (256, 4096, 256), (19, 8192, 256), (6, 2048, 0)])
 def test_rmsnorm_quantize_x(agemm, oracle, fmt, M, K, S):
     x = recipes.activations(M, K, seed=3000 + M + K + S, outlier_frac=0.005, outlier_gain=50.0)
     if M > 2:
@@ -195,13 +196,14 @@ def test_many_rows_unit_scale(agemm, oracle, fmt, M, K, S):
     compare("fused norm", q, sf, want)
 
 
-def test_dequantize_matches_oracle(agemm, oracle):
-    x = recipes.activations(12, 512, seed=77)
+@pytest.mark.parametrize("M,K,S", [(12, 512, 64), (300, 4096, 256), (7, 14336, 128)])
+def test_dequantize_matches_oracle(agemm, oracle, M, K, S):
+    x = recipes.activations(M, K, seed=77 + M)
     idx = recipes.reorder_index(x)
     for fmt in FMTS:
         gs = recipes.tensor_scale(x, fmt)
-        want = oracle.quantize_x(x, idx, 64, fmt, gs, want_dq=True)
-        q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), 64, fmt=fmt, global_scale=gs)
+        want = oracle.quantize_x(x, idx, S, fmt, gs, want_dq=True)
+        q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), S, fmt=fmt, global_scale=gs)
         assert np.array_equal(agemm.dequantize(q, sf, fmt=fmt).cpu().numpy(), want["dq"])
 
 
