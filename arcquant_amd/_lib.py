@@ -43,6 +43,8 @@ def lib() -> ctypes.CDLL:
     L.arcq_last_hip_error.restype = i
     L.arcq_prepare_stream.argtypes = [vp]
     L.arcq_prepare_stream.restype = i
+    L.arcq_release_stream.argtypes = [vp]
+    L.arcq_release_stream.restype = i
     L.arcq_group_size.argtypes = [i]
     L.arcq_group_size.restype = i
     L.arcq_codes_bytes.argtypes = [i, i, i]

@@ -31,7 +31,7 @@ from . import _lib
 from ._lib import FORMATS, ArcqError  # noqa: F401
 
 __all__ = ["matmul", "reorder_quantize_x", "reorder_quantize_w", "rmsnorm_quantize_x", "init_kv_i4", "append_kv_i4",
-           "batch_decode_i4", "swiglu_quantize_x", "tensor_scale", "prepare_stream", "dequantize", "check_index",
+           "batch_decode_i4", "swiglu_quantize_x", "tensor_scale", "prepare_stream", "release_stream", "dequantize", "check_index",
            "unpack_codes", "scale_values", "grouped_tensor_scale", "grouped_reorder_quantize_x",
            "grouped_swiglu_quantize_x", "grouped_matmul", "moe_route", "moe_combine", "matmul_swiglu",
            "grouped_matmul_swiglu", "interleave_gate_up"]
@@ -522,6 +522,15 @@ def prepare_stream(device=None) -> None:
     probe = torch.empty(0, device=dev)
     with _on_device(probe):
         _lib.check(_lib.lib().arcq_prepare_stream(_stream(probe)), "arcq_prepare_stream")
+
+
+def release_stream(stream=None) -> None:
+    """Free the library's scratch buffers of a torch stream (default: the current one) on its device
+    (arcq_release_stream): for streams about to be destroyed.  Never while a graph captured on the stream may
+    still be replayed -- the graph holds the buffers' addresses."""
+    st = torch.cuda.current_stream() if stream is None else stream
+    with torch.cuda.device(st.device):
+        _lib.check(_lib.lib().arcq_release_stream(ctypes.c_void_p(st.cuda_stream)), "arcq_release_stream")
 
 
 # The three INT4 KV-cache operators of the reference's module (kernels/src/bindings.cpp:576-578), so that a

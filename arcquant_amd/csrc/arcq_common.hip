@@ -64,6 +64,29 @@ void *stream_workspace(int kind, hipStream_t stream, int *status) {
   return p;
 }
 
+int release_stream_workspace(hipStream_t stream) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return note_hip_error(e);
+  void *ptr[kWsKinds] = {nullptr, nullptr, nullptr};
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    for (size_t i = 0; i < g_ws.size(); ++i)
+      if (g_ws[i].device == dev && g_ws[i].stream == stream) {
+        for (int k = 0; k < kWsKinds; ++k) ptr[k] = g_ws[i].ptr[k];
+        g_ws.erase(g_ws.begin() + (long)i);
+        break;
+      }
+  }
+  int rc = ARCQ_OK;
+  for (int k = 0; k < kWsKinds; ++k)
+    if (ptr[k]) {
+      e = hipFree(ptr[k]);  // waits for the device: no kernel still reads the buffer afterwards
+      if (e != hipSuccess) rc = note_hip_error(e);
+    }
+  return rc;
+}
+
 const Tuning &tuning() {
   static const Tuning t = [] {
     Tuning v;
@@ -107,7 +130,9 @@ int arcq_prepare_stream(void *stream) {
     int status = ARCQ_OK;
     if (!arcq::stream_workspace(kind, st, &status)) return status;
   }
-  return ARCQ_OK;
+  return arcq::noalloc_prepare();  // the fixed array of arcq_matmul_noalloc: its address on this device
 }
+
+int arcq_release_stream(void *stream) { return arcq::release_stream_workspace(static_cast<hipStream_t>(stream)); }
 
 }  // extern "C"

@@ -1250,7 +1250,7 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
   // (only while the two slices fit the 8 MiB array of the entry point that allocates nothing, which serves
   // every decode batch: N up to 32768 at 32 rows)
   const bool small_nv = fmt == ARCQ_FMT_NVFP4 && split_env == 0 && force < 0 && M >= 8 && M <= 32 && N >= 16384 && Kp < 8192 &&
-                        (size_t)2 * M * N * sizeof(float) <= ((size_t)8 << 20);
+                        (size_t)2 * M * N * sizeof(float) <= kNoAllocScratchBytes;
   if (split_env > 1) split = M <= 512 ? split_env : 0;
   else if (small_nv) split = 2;
   else if (split_env == 0 && force < 0 && M <= 64 && N <= 8192) {
@@ -1426,7 +1426,6 @@ int matmul_impl(const void *a_codes, const void *a_scales, const void *b_codes, 
 // that array, not a device address: its address on each device comes from hipGetSymbolAddress, once
 // per device, and only that pointer is handed to kernels.
 // ---------------------------------------------------------------------------------------------
-constexpr size_t kNoAllocScratchBytes = 8u << 20;
 constexpr int kNoAllocMaxDevices = 64;
 
 }  // namespace
@@ -1465,6 +1464,11 @@ float *noalloc_scratch(int *status) {
 }
 
 }  // namespace
+
+int noalloc_prepare() {
+  int status = ARCQ_OK;
+  return noalloc_scratch(&status) ? ARCQ_OK : status;
+}
 }  // namespace arcq
 
 extern "C" int arcq_matmul_noalloc(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales,

@@ -37,6 +37,16 @@ constexpr size_t kWorkspaceBytes[kWsKinds] = {256, 32u << 20, 8u << 20};
 // would break the capture), ARCQ_ERR_LAUNCH when the allocation fails.
 void *stream_workspace(int kind, hipStream_t stream, int *status);
 
+// Frees the buffers of (current device, stream) and forgets the pair; ARCQ_OK also when there were none.
+int release_stream_workspace(hipStream_t stream);
+
+// Size of the fixed device array behind arcq_matmul_noalloc.  The GEMM planner also reads it: the plans it
+// makes for decode batches must fit the array, so that arcq_matmul and arcq_matmul_noalloc serve the same shapes.
+constexpr size_t kNoAllocScratchBytes = 8u << 20;
+
+// Resolves the device address of that array on the current device (once per device; no allocation).
+int noalloc_prepare();
+
 // Overrides for tuning runs, read from the environment once, when the library is first used:
 //   ARCQ_GEMM_KERNEL=<WN><WM>   force a GEMM tile (84 / 82 = 256x256 / 256x128 as eight waves, 44, 42, 22, 21, 11; 214 / 224 = four-stage
 //                               ring; 1 = skinny, 0 = direct); a number the format has no kernel for is ignored

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t *y, con
 // ---------------------------------------------------------------------------------------------
 // Routing (model/qMixtralLayer.py:441-452: softmax over the experts in fp32, top-k, the k weights divided by
 // their sum and cast to the activations' type; :456-471 then walks the experts and the tokens routed to each).
-// Two launches replace a dozen of torch's: per token the choice and its weights, per (token, slot) pair its row
+// Two launches (three beyond 16384 tokens) replace a dozen of torch's: per token the choice and its weights, per (token, slot) pair its row
 // in the expert-sorted order (pairs of one expert in ascending pair number, as a stable sort by expert gives),
 // the expert segments, and the sorted views of token number and weight the grouped launches read.
 //
@@ -183,11 +183,70 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_choose_kernel(const v
   }
 }
 
+// Many tokens (more than kScanFromBlocks workgroups of the first launch): every workgroup of the placing launch
+// summing the whole histogram would be quadratic in the token count.  One workgroup turns the histograms
+// [blocks][E] into running sums over the earlier workgroups, expert by expert (a thread adds up a contiguous
+// run of workgroups, the runs' sums are scanned in LDS, the thread writes its run's prefixes back), and writes
+// the segments; the placing launch then reads E words per workgroup.
+constexpr int kScanThreads = 256;
+constexpr int kScanFromBlocks = 256;
+
+__global__ __launch_bounds__(kScanThreads) void moe_route_scan_kernel(int blocks, int E, int *hist, int *seg) {
+  __shared__ int part[kScanThreads];
+  __shared__ int total[kMaxExperts];
+  const int run = (blocks + kScanThreads - 1) / kScanThreads;
+  const int b0 = (int)threadIdx.x * run, b1 = min(blocks, b0 + run);
+  for (int e = 0; e < E; ++e) {
+    int sum = 0;
+    for (int b = b0; b < b1; ++b) sum += hist[(size_t)b * E + e];
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    for (int off = 1; off < kScanThreads; off <<= 1) {  // inclusive scan of the runs' sums
+      const int add = (int)threadIdx.x >= off ? part[threadIdx.x - off] : 0;
+      __syncthreads();
+      part[threadIdx.x] += add;
+      __syncthreads();
+    }
+    int before = part[threadIdx.x] - sum;
+    for (int b = b0; b < b1; ++b) {
+      const int v = hist[(size_t)b * E + e];
+      hist[(size_t)b * E + e] = before;
+      before += v;
+    }
+    if (threadIdx.x == kScanThreads - 1) total[e] = part[threadIdx.x];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < E; ++e) {
+      seg[e] = at;
+      at += total[e];
+    }
+    seg[E] = at;
+  }
+}
+
+template <bool SCANNED>
 __global__ __launch_bounds__(kRouteThreads) void moe_route_place_kernel(int T, int E, int top_k, const int *sel, const uint16_t *w,
                                                                         const int *hist, int64_t *position, int *seg, int *tok,
                                                                         uint16_t *ws) {
   __shared__ int start[kMaxExperts];  // first sorted row of this workgroup's pairs of expert e
   __shared__ int total[kMaxExperts], earlier[kMaxExperts];
+  if (SCANNED) {  // hist holds the sums over the earlier workgroups, seg is final
+    if ((int)threadIdx.x < E) start[threadIdx.x] = seg[threadIdx.x] + hist[(size_t)blockIdx.x * E + threadIdx.x];
+    __syncthreads();
+    const int t = blockIdx.x * kRouteThreads + threadIdx.x;
+    if (t >= T) return;
+    for (int j = 0; j < top_k; ++j) {
+      const size_t pair = (size_t)t * top_k + j;
+      if ((unsigned)sel[pair] >= (unsigned)E) continue;
+      const int64_t pos = start[sel[pair]] + position[pair];
+      position[pair] = pos;
+      tok[pos] = t;
+      ws[pos] = w[pair];
+    }
+    return;
+  }
   if (threadIdx.x < kMaxExperts) total[threadIdx.x] = earlier[threadIdx.x] = 0;
   __syncthreads();
   // The histograms [workgroups][E] were written on other XCDs and come from memory: a lane takes eight of
@@ -269,9 +328,17 @@ extern "C" int arcq_moe_route(const void *logits, int logits_f32, int tokens, in
   else { ARCQ_ROUTE(64) }
 #undef ARCQ_ROUTE
   ARCQ_HIP_TRY(hipGetLastError());
-  hipLaunchKernelGGL(moe_route_place_kernel, dim3(blocks), dim3(kRouteThreads), 0, st, tokens, experts, top_k, sel,
-                     static_cast<const uint16_t *>(weight), hist, position, seg_offsets, token_of_row,
-                     static_cast<uint16_t *>(weight_of_row));
+  if (blocks > kScanFromBlocks) {
+    hipLaunchKernelGGL(moe_route_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, blocks, experts, hist, seg_offsets);
+    ARCQ_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(moe_route_place_kernel<true>, dim3(blocks), dim3(kRouteThreads), 0, st, tokens, experts, top_k, sel,
+                       static_cast<const uint16_t *>(weight), hist, position, seg_offsets, token_of_row,
+                       static_cast<uint16_t *>(weight_of_row));
+  } else {
+    hipLaunchKernelGGL(moe_route_place_kernel<false>, dim3(blocks), dim3(kRouteThreads), 0, st, tokens, experts, top_k, sel,
+                       static_cast<const uint16_t *>(weight), hist, position, seg_offsets, token_of_row,
+                       static_cast<uint16_t *>(weight_of_row));
+  }
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }

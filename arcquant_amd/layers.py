@@ -693,14 +693,28 @@ class GraphedDecodeStep:
     The cache is shared by all layers of a model and must advance once per token, not once per layer:
     only the step with ``advance=True`` (the default for layer_idx 0) calls cache.begin_step(); the steps
     of the other layers run behind it on the advanced cache.  A caller that advances the cache itself
-    passes advance=False everywhere."""
+    passes advance=False everywhere.
 
-    def __init__(self, layer: LlamaDecoderLayer, cache, batch, hidden, layer_idx=0, warmup=3, advance=None):
+    All steps of a device are captured on ONE side stream (``stream=`` overrides it): the library's scratch
+    buffers belong to a (device, stream) pair and stay with a captured graph, and the steps of a model run one
+    after the other, so they can share one set (about 40 MiB) instead of holding one per layer."""
+
+    _capture_streams = {}
+
+    @classmethod
+    def capture_stream(cls, device):
+        device = torch.device(device)
+        key = (device.type, torch.cuda.current_device() if device.index is None else device.index)
+        if key not in cls._capture_streams:
+            cls._capture_streams[key] = torch.cuda.Stream(device=device)
+        return cls._capture_streams[key]
+
+    def __init__(self, layer: LlamaDecoderLayer, cache, batch, hidden, layer_idx=0, warmup=3, advance=None, stream=None):
         self.layer, self.cache, self.layer_idx = layer, cache, layer_idx
         self.advance = (layer_idx == 0) if advance is None else bool(advance)
         cache.external_step = True
         self.x = torch.zeros(batch, 1, hidden, dtype=torch.bfloat16, device=cache.device)
-        side = torch.cuda.Stream()
+        side = self.capture_stream(cache.device) if stream is None else stream
         side.wait_stream(torch.cuda.current_stream())
         saved = list(cache.lengths)
         # warm-up and capture run on a cache advanced by one token (the slot a real step writes), whichever

@@ -57,15 +57,21 @@ int arcq_last_hip_error(void);
  * (fp32 partial tiles, arcq_matmul on narrow layers with few rows), the split decode attention
  * (partial softmax sums, arcq_kv_decode_i4 with few sequences) and arcq_tensor_scale (two words).
  * The library keeps one buffer of each kind per (device, stream), allocated on the first call that
- * needs it and never freed; calls on one stream are serialised, so they never share a buffer with a
- * call on another stream.  An allocation cannot happen while the stream is being captured into a
+ * needs it and kept until arcq_release_stream or the end of the process (32 MiB + 8 MiB + 256 B when all
+ * three exist); calls on one stream are serialised, so they never share a buffer with a call on another
+ * stream.  An allocation cannot happen while the stream is being captured into a
  * graph: such a call returns ARCQ_ERR_WORKSPACE unless the stream has its buffers already.
- * arcq_prepare_stream allocates all three for (current device, stream) -- call it once before
- * capturing on that stream.  A graph replayed on another stream still uses the buffers of the stream
+ * arcq_prepare_stream allocates all three for (current device, stream), and resolves the address of
+ * arcq_matmul_noalloc's fixed array on that device -- call it once before capturing on that stream.  A graph replayed on another stream still uses the buffers of the stream
  * it was captured on.  (The reference keeps no state between calls: its CUTLASS GEMM has no split-K
  * and it computes tensor scales with torch, kernels/src/nvfp4.cu:35-132, model/qLlamaLayer.py:73-77.)
  */
 int arcq_prepare_stream(void *stream);
+/* Frees the scratch buffers of (current device, stream) and forgets the pair: call it before destroying a
+ * stream that ever ran one of the three kernels above (a later stream may get the same handle and would
+ * inherit the buffers otherwise), and never while a graph captured on that stream may still be replayed.
+ * Waits for the device.  ARCQ_OK also when the stream has no buffers.  No counterpart in the reference. */
+int arcq_release_stream(void *stream);
 
 /* Block size G of a format (16 / 32), or 0 for an unknown format. */
 int arcq_group_size(int fmt);
@@ -187,8 +193,9 @@ int arcq_matmul_add(const void *a_codes, const void *a_scales, const void *b_cod
  *   - All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams,
  *     two threads) race.  The array keeps the last call's contents; every word a call reads back it has
  *     written first, so nothing needs clearing.
- *   - The first call on a device resolves the array's address (hipGetSymbolAddress); make one call, of this
- *     or any other entry point after loading the library, before a capture.
+ *   - The array's address on a device is resolved (hipGetSymbolAddress, no allocation) by arcq_prepare_stream,
+ *     or else by the first call of this entry point on that device whose plan cuts K: do one of the two
+ *     before a capture.
  */
 int arcq_matmul_noalloc(const void *a_codes, const void *a_scales, const void *b_codes, const void *b_scales, int M, int N,
                         int Kp, int fmt, float alpha, const float *d_alpha_a, const float *d_alpha_b, void *c,

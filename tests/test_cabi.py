@@ -111,3 +111,21 @@ def test_grouped_entry_points_reject_bad_arguments():
     assert mr(ok, 0, 4096, 8, 2, ok, ok, ok, ok, ok, ok, ok, 16, None) == 7                   # workspace too small
     assert L.arcq_stream_probe_variants() >= 2
     assert L.arcq_stream_probe_variant(ok, ok, 1024, 512, 99, None) == 2
+
+
+def test_decode_batches_fit_the_no_alloc_array():
+    """arcq_matmul and arcq_matmul_noalloc share one planner: every decode batch (M <= 64) of the Llama-3-8B
+    projection shapes must get a plan whose split-K partial tiles fit the fixed array, in both formats"""
+    L = _lib.lib()
+    limit = L.arcq_matmul_noalloc_limit()
+    assert limit == 8 << 20
+    for fmt in (0, 1):
+        for N, K in ((6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)):
+            for S in (64, 128, 256):
+                for M in range(1, 65):
+                    need = L.arcq_matmul_scratch_bytes(M, N, K + S, fmt)
+                    assert need <= limit, (fmt, M, N, K + S, need)
+
+
+def test_release_stream_without_buffers_needs_no_gpu_work():
+    assert hasattr(_lib.lib(), "arcq_release_stream")

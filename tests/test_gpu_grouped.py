@@ -288,7 +288,8 @@ print("OK")
     assert r.returncode == 0 and "OK" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
 
 
-@pytest.mark.parametrize("T,E,k,dtype", [(4096, 8, 2, torch.bfloat16), (300, 8, 2, torch.float32), (1000, 16, 4, torch.bfloat16),
+@pytest.mark.parametrize("T,E,k,dtype", [(4096, 8, 2, torch.bfloat16), (16384, 8, 2, torch.bfloat16), (16385, 8, 2, torch.bfloat16),
+                                         (70001, 8, 2, torch.bfloat16), (40000, 64, 6, torch.float32), (300, 8, 2, torch.float32), (1000, 16, 4, torch.bfloat16),
                                          (1, 8, 2, torch.bfloat16), (777, 64, 8, torch.float32), (50, 5, 2, torch.bfloat16),
                                          (513, 3, 3, torch.float32)])
 def test_moe_route_matches_torch(agemm, T, E, k, dtype):

@@ -74,3 +74,39 @@ def test_noalloc_without_scratch_and_beyond_the_limit(L):
     ok = ctypes.c_void_p(0x1000)                                   # never dereferenced: the call returns first
     assert L.arcq_matmul_noalloc(ok, ok, ok, ok, M, N, Kp, 0, 1.0, None, None, ok, None) == 7
     assert b"scratch" in L.arcq_status_string(7)
+
+
+def test_noalloc_allocates_nothing(L):
+    """What the entry point is named for: on a stream the library has never seen (no scratch buffers of its
+    own), a call whose plan cuts K leaves the device's free memory where it was -- arcq_matmul on such a stream
+    takes 32 MiB for its partial tiles -- and a released stream starts from nothing again."""
+    from arcquant_amd import agemm
+    M, N, K, S, fid = 64, 4096, 14336, 256, 1
+    ops = operands(agemm, M, N, K, S, "MXFP4", seed=5)
+    rc, want = call(L.arcq_matmul, ops, M, N, K + S, fid)            # kernels loaded, torch's pools warm
+    assert rc == 0
+    torch.cuda.synchronize()
+    fresh = torch.cuda.Stream()
+    c = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    a, sfa, b, sfb = ops
+    handle = ctypes.c_void_p(fresh.cuda_stream)
+    fresh.wait_stream(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    rc = L.arcq_matmul_noalloc(a.data_ptr(), sfa.data_ptr(), b.data_ptr(), sfb.data_ptr(), M, N, K + S, fid, 0.5, None, None,
+                               c.data_ptr(), handle)
+    torch.cuda.synchronize()
+    free1 = torch.cuda.mem_get_info()[0]
+    assert rc == 0 and torch.equal(c, want)
+    assert free0 - free1 < (1 << 20), (free0, free1)
+    # the allocating entry point on the same stream does take its buffer, and arcq_release_stream gives it back
+    rc = L.arcq_matmul(a.data_ptr(), sfa.data_ptr(), b.data_ptr(), sfb.data_ptr(), M, N, K + S, fid, 0.5, None, None,
+                       c.data_ptr(), handle)
+    torch.cuda.synchronize()
+    free2 = torch.cuda.mem_get_info()[0]
+    assert rc == 0 and torch.equal(c, want)
+    assert free1 - free2 >= (32 << 20) - (1 << 20), (free1, free2)
+    assert L.arcq_release_stream(handle) == 0
+    free3 = torch.cuda.mem_get_info()[0]
+    assert free3 - free2 >= (32 << 20) - (1 << 20), (free2, free3)
+    assert L.arcq_release_stream(handle) == 0                         # nothing left: still fine
