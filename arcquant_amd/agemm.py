@@ -166,7 +166,7 @@ def swiglu_quantize_x(gate, up, reorder_index, KE, *, fmt="NVFP4", global_scale=
     ld = gate.stride(0) if M > 1 else K
     KE = int(KE)
     G = _lib.GROUP_SIZE[f]
-    if K % 32 or K < 32 or K > 16384 or KE < 0 or KE > K or KE % G or reorder_index.numel() != K or ld % 8:
+    if K % 32 or K < 32 or K > 32736 or KE < 0 or KE > K or KE % G or reorder_index.numel() != K or ld % 8:
         raise RuntimeError(f"Value error in swiglu_quantize_x: K={K}, KE={KE}, row stride {ld} not supported for {fmt}")
     want_scale = isinstance(global_scale, str)
     with _on_device(gate):
@@ -293,7 +293,7 @@ def _grouped_quantize(gate, up, seg, reorder_index, KE, fmt, global_scales):
     G = _lib.GROUP_SIZE[f]
     if tuple(reorder_index.shape) != (E, K) or reorder_index.device != gate.device:
         raise RuntimeError(f"reorder_index must be int16 [{E}, {K}] on the operands' device")
-    if K % 32 or K < 32 or K > 16384 or KE < 0 or KE > K or KE % G:
+    if K % 32 or K < 32 or K > 32736 or KE < 0 or KE > K or KE % G:
         raise RuntimeError(f"Value error in grouped quantizer: K={K}, KE={KE} not supported for {fmt}")
     if global_scales is not None:
         _require(global_scales, "global_scales", torch.float32, 1)

@@ -20,6 +20,8 @@ from typing import Dict
 import torch
 
 NAME_TEMPLATE = "layers.{}.{}.{}.input"   # layer index, block ('self_attn' / 'mlp'), projection
+# a Mixtral expert's linears (model/qMixtralLayer.py:488): layer index, expert index, projection ('w1' / 'w2' / 'w3')
+MOE_NAME_TEMPLATE = "layers.{}.block_sparse_moe.experts.{}.{}.input"
 
 
 def reorder_index_from_stat(stat: torch.Tensor) -> torch.Tensor:

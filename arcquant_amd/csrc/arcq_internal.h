@@ -52,7 +52,8 @@ int noalloc_prepare();
 //                               ring; 1 = skinny, 0 = direct); a number the format has no kernel for is ignored
 //   ARCQ_GEMM_SPLITK=<slices>   force split-K for M <= 512 (1 = never split)
 //   ARCQ_QUANT_GRID=<n>         workgroups of the row quantizers
-//   ARCQ_QUANT_KERNEL=<1|2>     1 = never, 2 = always take the wave-per-row quantizer where it has an instance
+//   ARCQ_QUANT_KERNEL=<1|2|3>   1 = never, 2 = always take the wave-per-row quantizer where it has an instance;
+//                               3 = the four-units-per-thread kernel of the rows beyond 16384 channels from 1024 channels on
 //   ARCQ_KV_DECODE_SPLITS=<n>   ranges per sequence of the decode attention
 // Unset (the normal case) every field keeps the value below and the dispatch is the measured one.
 struct Tuning {

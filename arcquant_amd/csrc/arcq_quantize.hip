@@ -367,6 +367,64 @@ __device__ __forceinline__ void unit_exact(const uint32_t (&yv)[16], float g, ui
   }
 }
 
+// One unit's arithmetic, shared by the row kernels below: yv holds the unit's 16 gathered bf16 values as fp32
+// bits (all zero in a lane without a unit).  Returns codes and scale byte of the unit (pk, sb) and, for a unit
+// among the last select_num channels of an activation (tail), those of its residual block (pk2, sb2; for
+// weights and elsewhere a copy of pk, sb).  Every lane of the wave must call it (MXFP4 exchanges the maxima
+// of the two halves of a 32-block between neighbouring lanes).
+template <int FMT, int MODE, bool SCALED>
+__device__ __forceinline__ void quantize_unit(const uint32_t (&yv)[16], bool active, bool tail, float g, float rg, bool g_odd,
+                                              bool coarse, uint2 &pk, uint32_t &sb, uint2 &pk2, uint32_t &sb2) {
+  float y[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) y[i] = u2f(yv[i]);
+  if (SCALED) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) y[i] = div_bf16_by(y[i], g, rg);
+  }
+  float s;
+  const float amax = unit_amax3<FMT>(y);
+  const float t = div6_any(amax);
+  sb = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t, &s) : ue8m0_scale(t, &s);
+  bool redo = false;  // SCALED only: this unit needs unit_exact
+  if (coarse) {
+    pk = encode_unit_coarse(y, scale_rcp<FMT>(s));
+    if (SCALED) redo = amax_needs_exact(amax) || g_odd;
+  } else {
+    pk = encode_unit_two_sided(y, s, scale_rcp<FMT>(s));
+    redo = amax_needs_exact(amax) || g_odd;
+  }
+  pk2 = pk;
+  sb2 = sb;
+  if (MODE != MODE_W && tail) {
+    float e[16];
+    decode_unit(pk, e);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) e[i] = __builtin_fmaf(-e[i], s, y[i]);  // q*s is exact: the fp32 residual y - q*s
+    float s2;
+    const float amax2 = unit_amax3<FMT>(e);
+    const float t2 = div6_any(amax2);
+    sb2 = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t2, &s2) : ue8m0_scale(t2, &s2);
+    if (coarse) {
+      pk2 = encode_unit_coarse(e, scale_rcp<FMT>(s2));
+      if (SCALED) redo = amax_needs_exact(amax2) || redo;
+    } else {
+      pk2 = encode_unit_two_sided(e, s2, scale_rcp<FMT>(s2));
+      redo = amax_needs_exact(amax2) || redo;
+    }
+  }
+  if (SCALED && FMT == ARCQ_FMT_MXFP4) redo = __shfl_xor((int)redo, 1) != 0 || redo;  // both halves of a 32-block
+  if (SCALED && redo && active) {
+    if (MODE != MODE_W && tail) {
+      unit_exact<FMT, true>(yv, g, &pk, &sb, &pk2, &sb2);
+    } else {
+      unit_exact<FMT, false>(yv, g, &pk, &sb, &pk2, &sb2);
+      pk2 = pk;
+      sb2 = sb;
+    }
+  }
+}
+
 template <int FMT, int MODE, bool SCALED, bool GROUPED = false>
 __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p) {
   extern __shared__ uint4 smem[];
@@ -546,59 +604,12 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
       for (int i = 0; i < 16; ++i) asm volatile("ds_read_u16_d16_hi %0, %1" : "+v"(yv[i]) : "v"(addr[i]) : "memory");
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
-    float y[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) y[i] = u2f(yv[i]);
-
     uint8_t *crow = p.codes + (size_t)r * (Kp >> 1);
     uint8_t *srow = p.scales + (size_t)r * (Kp / G);
-    if (SCALED) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) y[i] = div_bf16_by(y[i], g, rg);
-    }
-    float s;
-    const float amax = unit_amax3<FMT>(y);
-    const float t = div6_any(amax);
-    uint32_t sb = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t, &s) : ue8m0_scale(t, &s);
-    uint2 pk;
-    bool redo = false;  // SCALED only: this unit needs unit_exact
-    if (coarse) {
-      pk = encode_unit_coarse(y, scale_rcp<FMT>(s));
-      if (SCALED) redo = amax_needs_exact(amax) || g_odd;
-    } else {
-      pk = encode_unit_two_sided(y, s, scale_rcp<FMT>(s));
-      redo = amax_needs_exact(amax) || g_odd;
-    }
     const bool tail = active && tid >= tail0;
-    uint2 pk2 = pk;
-    uint32_t sb2 = sb;
-    if (MODE != MODE_W && tail) {
-      float e[16];
-      decode_unit(pk, e);
-#pragma unroll
-      for (int i = 0; i < 16; ++i) e[i] = __builtin_fmaf(-e[i], s, y[i]);  // q*s is exact: the fp32 residual y - q*s
-      float s2;
-      const float amax2 = unit_amax3<FMT>(e);
-      const float t2 = div6_any(amax2);
-      sb2 = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t2, &s2) : ue8m0_scale(t2, &s2);
-      if (coarse) {
-        pk2 = encode_unit_coarse(e, scale_rcp<FMT>(s2));
-        if (SCALED) redo = amax_needs_exact(amax2) || redo;
-      } else {
-        pk2 = encode_unit_two_sided(e, s2, scale_rcp<FMT>(s2));
-        redo = amax_needs_exact(amax2) || redo;
-      }
-    }
-    if (SCALED && FMT == ARCQ_FMT_MXFP4) redo = __shfl_xor((int)redo, 1) != 0 || redo;  // both halves of a 32-block
-    if (SCALED && redo && active) {
-      if (MODE != MODE_W && tail) {
-        unit_exact<FMT, true>(yv, g, &pk, &sb, &pk2, &sb2);
-      } else {
-        unit_exact<FMT, false>(yv, g, &pk, &sb, &pk2, &sb2);
-        pk2 = pk;
-        sb2 = sb;
-      }
-    }
+    uint2 pk, pk2;
+    uint32_t sb, sb2;
+    quantize_unit<FMT, MODE, SCALED>(yv, active, tail, g, rg, g_odd, coarse, pk, sb, pk2, sb2);
     // The next row's registers are taken over before this row's stores are issued: the wait for
     // the prefetch (in flight since the top of the iteration) then stands in front of the stores, and
     // the top of the next iteration has no memory operation of this one left to wait for.
@@ -613,6 +624,153 @@ __global__ __launch_bounds__(1024) void quantize_rows_unit_kernel(QuantParams p)
     if (active) {
       store_unit<FMT>(crow, srow, tid, pk, sb);
       if (tail) store_unit<FMT>(crow, srow, nunits + (tid - tail0), pk2, sb2);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rows of more than 16384 channels (the reference's dedicated shapes: 18944, 27648, 28672;
+// kernels/src/bindings.cpp:141-160, down.cu:71-233, reorder.cu:380-555), every mode but the fused norm.
+// A thread per unit would need more than 1024 threads and a row of up to 64 KB leaves room for one such
+// workgroup per CU, which would then load, gather and store in turns.  Here a thread owns FOUR units
+// (u = tid + h * blockDim, so that a wave's code stores stay contiguous), a workgroup is K/64 threads
+// (at most 512) and two of them fit a CU: one loads its next row while the other encodes.  The channel
+// order stays in registers as the 16-bit indices themselves (eight registers per unit); a gather address
+// is one multiply-add away.  The arithmetic per unit is quantize_unit, as in the kernel above.
+// ---------------------------------------------------------------------------------------------
+// slot address of channel `half` (0 / 1) of an index pair: base + 2 * index, one instruction
+template <int HALF>
+__device__ __forceinline__ uint32_t gather_addr(uint32_t pair, uint32_t base) {
+  uint32_t a;
+  if (HALF == 0)
+    asm("v_mad_u32_u16 %0, %1, 2, %2" : "=v"(a) : "v"(pair), "v"(base));
+  else
+    asm("v_mad_u32_u16 %0, %1, 2, %2 op_sel:[1,0,0,0]" : "=v"(a) : "v"(pair), "v"(base));
+  return a;
+}
+
+constexpr int kWideUnits = 4;
+
+template <int FMT, int MODE, bool SCALED, bool GROUPED = false>
+__global__ __launch_bounds__(512, 4) void quantize_rows_wide_kernel(QuantParams p) {
+  extern __shared__ uint4 smem[];
+  static_assert(MODE != MODE_NORM, "the fused norm has no rows this long");
+  constexpr int G = FMT == ARCQ_FMT_NVFP4 ? 16 : 32;
+  const int K = p.K, S = p.S, Kp = K + S;
+  uint16_t *row = reinterpret_cast<uint16_t *>(smem);
+  const uint32_t row_addr = (uint32_t)reinterpret_cast<uintptr_t>(row);
+  const int T = blockDim.x, nwaves = T >> 6;
+  int tid = threadIdx.x + 64 * (int)(blockIdx.x % (unsigned)nwaves);  // the waves with residual units rotate over the SIMDs
+  if (tid >= T) tid -= T;
+  const int nunits = K >> 4, nchunks = K >> 3, tail0 = (K - S) >> 4;
+  const size_t ldx = MODE == MODE_SWIGLU ? (size_t)p.ldx : (size_t)K;
+
+  float g = SCALED ? (p.d_gscale && !GROUPED ? *p.d_gscale : p.gscale) : 1.0f;
+  float rg = SCALED ? 1.0f / g : 1.0f;
+  bool g_odd = SCALED && !(fabsf(g) >= 0x1p-60f && fabsf(g) <= 0x1p+60f);
+  bool coarse = !SCALED || (f2u(g) & 0x7fffffu) == 0u;
+
+  uint32_t iw[kWideUnits][8];
+  auto load_order = [&](const int16_t *idx) {
+#pragma unroll
+    for (int h = 0; h < kWideUnits; ++h) {
+      const int u = tid + h * T;
+      uint4 i0 = make_uint4(0, 0, 0, 0), i1 = i0;
+      if (u < nunits) {
+        i0 = reinterpret_cast<const uint4 *>(idx)[2 * u];
+        i1 = reinterpret_cast<const uint4 *>(idx)[2 * u + 1];
+      }
+      iw[h][0] = i0.x, iw[h][1] = i0.y, iw[h][2] = i0.z, iw[h][3] = i0.w;
+      iw[h][4] = i1.x, iw[h][5] = i1.y, iw[h][6] = i1.z, iw[h][7] = i1.w;
+    }
+  };
+  if (!GROUPED) load_order(p.idx);
+  int seg_cur = -1, seg_end = 0;
+  uint32_t yv[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) yv[i] = 0u;  // low halves stay zero: only d16_hi loads write these
+
+  for (int r = blockIdx.x; r < p.rows; r += gridDim.x) {
+    if (GROUPED && r >= seg_end) {  // workgroup-uniform; once per segment at most (rows are sorted)
+      while (seg_cur + 1 < p.n_seg && r >= seg_end) {
+        ++seg_cur;
+        seg_end = p.seg[seg_cur + 1];
+      }
+      if (r >= seg_end) break;
+      load_order(p.idx + (size_t)seg_cur * K);
+      if (SCALED) {
+        g = p.d_gscale[seg_cur];
+        rg = 1.0f / g;
+        g_odd = !(fabsf(g) >= 0x1p-60f && fabsf(g) <= 0x1p+60f);
+        coarse = (f2u(g) & 0x7fffffu) == 0u;
+      }
+    }
+    // the row, natural order: 2 * kWideUnits 16-byte chunks per thread, all in flight at once (SwiGLU, which
+    // reads two rows: in two halves)
+    const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (size_t)r * ldx);
+    const uint4 *usrc = MODE == MODE_SWIGLU ? reinterpret_cast<const uint4 *>(p.up + (size_t)r * ldx) : nullptr;
+    constexpr int kParts = MODE == MODE_SWIGLU ? 2 : 1, kPer = 2 * kWideUnits / kParts;
+    // Everything derived from the thread number below (chunk and unit offsets, their bounds checks) is the same
+    // for every row; hoisted out of the row loop it would stay in some forty registers across the encode.
+    // The thread number is therefore made opaque once per row and once per unit.
+    int tid_r = tid;
+    asm volatile("" : "+v"(tid_r));
+#pragma unroll
+    for (int part = 0; part < kParts; ++part) {
+      uint4 q[kPer], uq[kPer];
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int c = tid_r + (part * kPer + j) * T;
+        q[j] = make_uint4(0, 0, 0, 0);
+        uq[j] = q[j];
+        if (c < nchunks) {
+          q[j] = src[c];
+          if (MODE == MODE_SWIGLU) uq[j] = usrc[c];
+        }
+      }
+      if (part == 0) lds_barrier();  // the previous row's gathers are over (the loads above are already on their way)
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const int c = tid_r + (part * kPer + j) * T;
+        if (MODE == MODE_SWIGLU)
+          q[j] = make_uint4(swiglu_pair(q[j].x, uq[j].x), swiglu_pair(q[j].y, uq[j].y), swiglu_pair(q[j].z, uq[j].z),
+                            swiglu_pair(q[j].w, uq[j].w));
+        if (c < nchunks) reinterpret_cast<uint4 *>(row)[c] = q[j];
+      }
+    }
+    lds_barrier();
+
+    uint8_t *crow = p.codes + (size_t)r * (Kp >> 1);
+    uint8_t *srow = p.scales + (size_t)r * (Kp / G);
+#pragma unroll
+    for (int h = 0; h < kWideUnits; ++h) {
+      if (h * T >= nunits) break;  // workgroup-uniform: nobody has a unit in this round
+      int u = tid + h * T;
+      asm volatile("" : "+v"(u));
+      const bool active = u < nunits;  // a lane without a unit keeps the previous unit's values: nothing of it is stored
+      if (active) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          // (volatile: the addresses do not depend on the row, and hoisted out of the row loop they would
+          // occupy 64 registers)
+          uint32_t a0, a1;
+          asm volatile("v_mad_u32_u16 %0, %1, 2, %2" : "=v"(a0) : "v"(iw[h][j]), "v"(row_addr));
+          asm volatile("v_mad_u32_u16 %0, %1, 2, %2 op_sel:[1,0,0,0]" : "=v"(a1) : "v"(iw[h][j]), "v"(row_addr));
+          asm volatile("ds_read_u16_d16_hi %0, %1" : "+v"(yv[2 * j]) : "v"(a0) : "memory");
+          asm volatile("ds_read_u16_d16_hi %0, %1" : "+v"(yv[2 * j + 1]) : "v"(a1) : "memory");
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(yv[i]));  // read after the wait above
+      const bool tail = active && u >= tail0;
+      uint2 pk, pk2;
+      uint32_t sb, sb2;
+      quantize_unit<FMT, MODE, SCALED>(yv, active, tail, g, rg, g_odd, coarse, pk, sb, pk2, sb2);
+      if (active) {
+        store_unit<FMT>(crow, srow, u, pk, sb);
+        if (tail) store_unit<FMT>(crow, srow, nunits + (u - tail0), pk2, sb2);
+      }
     }
   }
 }
@@ -657,17 +815,6 @@ __device__ __forceinline__ void row_dma(const void *row, int lane, uint32_t lds_
     if (4 * h + 2 < NCH) row_dma16<2048>(gh, lb);
     if (4 * h + 3 < NCH) row_dma16<3072>(gh, lb);
   }
-}
-
-// slot address of channel `half` (0 / 1) of an index pair: base + 2 * index, one instruction
-template <int HALF>
-__device__ __forceinline__ uint32_t gather_addr(uint32_t pair, uint32_t base) {
-  uint32_t a;
-  if (HALF == 0)
-    asm("v_mad_u32_u16 %0, %1, 2, %2" : "=v"(a) : "v"(pair), "v"(base));
-  else
-    asm("v_mad_u32_u16 %0, %1, 2, %2 op_sel:[1,0,0,0]" : "=v"(a) : "v"(pair), "v"(base));
-  return a;
 }
 
 __device__ __forceinline__ void gather16(uint32_t (&yv)[16], const uint32_t (&addr)[16]) {
@@ -1038,6 +1185,23 @@ int launch_quantize_unit(const QuantParams &p, hipStream_t stream) {
   return ARCQ_OK;
 }
 
+template <int FMT, int MODE, bool SCALED, bool GROUPED = false>
+int launch_quantize_wide(const QuantParams &p, hipStream_t stream) {
+  const int threads = (((p.K >> 4) + 4 * 64 - 1) / (4 * 64)) * 64;  // four units per thread, whole waves
+  const size_t lds = (size_t)p.K * 2;
+  auto kern = quantize_rows_wide_kernel<FMT, MODE, SCALED, GROUPED>;
+  if (lds > 64 * 1024 - 512)
+    ARCQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  // as many workgroups as the chip holds at once: four waves per SIMD by registers, 160 KB of LDS per CU
+  const int by_waves = 16 / (threads / 64), by_lds = (int)((160 * 1024) / (lds + 256));
+  int grid = 256 * std::max(1, std::min(by_waves, by_lds));
+  if (tuning().quant_grid > 0) grid = tuning().quant_grid;
+  if (grid > p.rows) grid = p.rows;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, stream, p);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
 template <int FMT, int MODE, int KU>
 int launch_quantize_wave(const QuantParams &p, hipStream_t stream) {
   constexpr int K = 1024 * KU;
@@ -1217,6 +1381,16 @@ int quantize_entry(int mode, const void *x, const void *gamma, float eps, int ro
   p.up = nullptr;
   p.ldx = K;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // rows beyond what a thread per unit covers: four units per thread, two workgroups per CU
+  if (mode != MODE_NORM && (K > 16384 || (tuning().quant_kernel == 3 && K >= 1024))) {
+    const bool unit = !d_gscale && gscale == 1.0f;
+#define ARCQ_WIDE(F)                                                                                         \
+    if (mode == MODE_X) return unit ? launch_quantize_wide<F, MODE_X, false>(p, st) : launch_quantize_wide<F, MODE_X, true>(p, st); \
+    return unit ? launch_quantize_wide<F, MODE_W, false>(p, st) : launch_quantize_wide<F, MODE_W, true>(p, st);
+    if (fmt == ARCQ_FMT_NVFP4) { ARCQ_WIDE(ARCQ_FMT_NVFP4) }
+    ARCQ_WIDE(ARCQ_FMT_MXFP4)
+#undef ARCQ_WIDE
+  }
   // tensor scale known on the host to be 1: operands are exactly bf16 -> fast kernels
   if (!d_gscale && gscale == 1.0f && K <= 16384) {
     // fused norm over many rows of a hidden size up to 4096: a wave per row, sixteen rows per CU at a time (4096
@@ -1259,7 +1433,7 @@ int swiglu_entry(const void *gate, const void *up, int ld, int rows, int K, cons
                  float gscale, const float *d_gscale, void *codes, void *scales, void *stream) {
   if (fmt != ARCQ_FMT_NVFP4 && fmt != ARCQ_FMT_MXFP4) return ARCQ_ERR_FORMAT;
   const int G = arcq_group_size(fmt);
-  if (rows < 0 || K < 32 || K % 32 != 0 || K > 16384 || S < 0 || S > K || S % G != 0 || ld < K || ld % 8 != 0)
+  if (rows < 0 || K < 32 || K % 32 != 0 || K > 32736 || S < 0 || S > K || S % G != 0 || ld < K || ld % 8 != 0)
     return ARCQ_ERR_SHAPE;
   if (rows == 0) return ARCQ_OK;
   if (!gate || !up || !idx || !codes || !scales) return ARCQ_ERR_NULL;
@@ -1281,6 +1455,13 @@ int swiglu_entry(const void *gate, const void *up, int ld, int rows, int K, cons
   p.inv_k = 0.0;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool unit = !d_gscale && gscale == 1.0f;
+  if (K > 16384 || (tuning().quant_kernel == 3 && K >= 1024)) {
+    if (fmt == ARCQ_FMT_NVFP4)
+      return unit ? launch_quantize_wide<ARCQ_FMT_NVFP4, MODE_SWIGLU, false>(p, st)
+                  : launch_quantize_wide<ARCQ_FMT_NVFP4, MODE_SWIGLU, true>(p, st);
+    return unit ? launch_quantize_wide<ARCQ_FMT_MXFP4, MODE_SWIGLU, false>(p, st)
+                : launch_quantize_wide<ARCQ_FMT_MXFP4, MODE_SWIGLU, true>(p, st);
+  }
   if (fmt == ARCQ_FMT_NVFP4)
     return unit ? launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_SWIGLU, false>(p, st)
                 : launch_quantize_unit<ARCQ_FMT_NVFP4, MODE_SWIGLU, true>(p, st);
@@ -1294,7 +1475,7 @@ int grouped_quantize_entry(int mode, const void *x, const void *up, int ld, int 
                            void *stream) {
   if (fmt != ARCQ_FMT_NVFP4 && fmt != ARCQ_FMT_MXFP4) return ARCQ_ERR_FORMAT;
   const int G = arcq_group_size(fmt);
-  if (rows < 0 || n_seg < 1 || K < 32 || K % 32 != 0 || K > 16384 || S < 0 || S > K || S % G != 0 || ld < K || ld % 8 != 0)
+  if (rows < 0 || n_seg < 1 || K < 32 || K % 32 != 0 || K > 32736 || S < 0 || S > K || S % G != 0 || ld < K || ld % 8 != 0)
     return ARCQ_ERR_SHAPE;
   if (rows == 0) return ARCQ_OK;
   if (!x || !seg || !idx || !codes || !scales || (mode == MODE_SWIGLU && !up)) return ARCQ_ERR_NULL;
@@ -1318,6 +1499,17 @@ int grouped_quantize_entry(int mode, const void *x, const void *up, int ld, int 
   p.n_seg = n_seg;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool unit = d_gscales == nullptr;
+  if (K > 16384) {
+    if (mode == MODE_X && ld != K) return ARCQ_ERR_SHAPE;
+#define ARCQ_WIDE_G(F, MD) return unit ? launch_quantize_wide<F, MD, false, true>(p, st) : launch_quantize_wide<F, MD, true, true>(p, st);
+    if (mode == MODE_X) {
+      if (fmt == ARCQ_FMT_NVFP4) { ARCQ_WIDE_G(ARCQ_FMT_NVFP4, MODE_X) }
+      ARCQ_WIDE_G(ARCQ_FMT_MXFP4, MODE_X)
+    }
+    if (fmt == ARCQ_FMT_NVFP4) { ARCQ_WIDE_G(ARCQ_FMT_NVFP4, MODE_SWIGLU) }
+    ARCQ_WIDE_G(ARCQ_FMT_MXFP4, MODE_SWIGLU)
+#undef ARCQ_WIDE_G
+  }
   if (mode == MODE_X) {
     if (ld != K) return ARCQ_ERR_SHAPE;
     if (fmt == ARCQ_FMT_NVFP4)

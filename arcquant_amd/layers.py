@@ -245,7 +245,7 @@ class LlamaMLP(nn.Module):
                                                global_scale=scale if nv else None)
             return self.down_proj((qx, sfx, scale, x[3], x[4]), residual)
         gu = self.gate_up_proj(x)
-        if self.inter <= 16384 and self.inter % 32 == 0:
+        if self.inter <= 32736 and self.inter % 32 == 0:
             return self.down_proj(swiglu_quantize_tokens(gu, self.inter, self.down_reorder_index, sel, self.quant_type),
                                   residual)
         t = F.silu(gu[..., :self.inter]) * gu[..., self.inter:]
@@ -468,13 +468,16 @@ class QLlamaDecoderLayer(nn.Module):
     NVFP4 tensor scale max|x|/2688 of its input, as model/qLlamaLayer.py:73-86 does; fuse_norm=True swaps
     in the fused RMSNorm -> quantize operator (tensor scale 1: benchmarks/modeling_arc.py:211-227)."""
 
+    attention_class = QLlamaAttention
+    mlp_class = QLlamaMLP
+
     def __init__(self, linears, norm_weights, eps, num_heads, num_kv_heads, select_nums, reorder_index, layer_idx,
                  quant_type="NVFP4", fuse_norm=False):
         super().__init__()
-        self.self_attn = QLlamaAttention(linears["q_proj"], linears["k_proj"], linears["v_proj"], linears["o_proj"],
-                                         num_heads, num_kv_heads, select_nums, reorder_index, layer_idx, quant_type)
-        self.mlp = QLlamaMLP(linears["gate_proj"], linears["up_proj"], linears["down_proj"], select_nums,
-                             reorder_index, layer_idx, quant_type)
+        self.self_attn = self.attention_class(linears["q_proj"], linears["k_proj"], linears["v_proj"], linears["o_proj"],
+                                              num_heads, num_kv_heads, select_nums, reorder_index, layer_idx, quant_type)
+        self.mlp = self.mlp_class(linears["gate_proj"], linears["up_proj"], linears["down_proj"], select_nums,
+                                  reorder_index, layer_idx, quant_type)
         self.quant_type = quant_type
         self.layer_idx = layer_idx
         if fuse_norm:
@@ -534,7 +537,7 @@ class MixtralExpertMLP(nn.Module):
                                                global_scale=scale if nv else None)
             return self.w2((qx, sfx, scale, None, t.shape[0]))
         h = self.w13(xq)
-        if self.ffn <= 16384 and self.ffn % 32 == 0:
+        if self.ffn <= 32736 and self.ffn % 32 == 0:
             return self.w2(swiglu_quantize_tokens(h, self.ffn, self.w2_reorder_index, self.w2.select_num,
                                                   self.quant_type))
         t = F.silu(h[:, :self.ffn]) * h[:, self.ffn:]
@@ -566,7 +569,7 @@ class MixtralSparseMoeBlock(nn.Module):
                    for ex in experts)
         kp13, kp2 = 2 * e0.w13.W.shape[1], 2 * e0.w2.W.shape[1]
         self.grouped = bool(grouped) and same and kp13 % 128 == 0 and kp2 % 128 == 0 and min(kp13, kp2) >= 512 and \
-            e0.ffn <= 16384 and e0.ffn % 32 == 0 and e0.w13.in_features <= 16384
+            e0.ffn <= 32736 and e0.ffn % 32 == 0 and e0.w13.in_features <= 32736
         if self.grouped:
             self.quant_type, self.ffn, self.interleaved = e0.quant_type, e0.ffn, e0.interleaved
             for name in ("w13", "w2"):
@@ -681,6 +684,133 @@ def build_mixtral_block(hidden=4096, ffn=14336, num_experts=8, top_k=2, select_n
         experts.append(MixtralExpertMLP(w1, w3, w2, select_num, i_in, i_w2, quant_type, interleave=interleave))
         del w1, w3, w2
     return MixtralSparseMoeBlock(gate, experts, top_k, grouped=grouped)
+
+
+class QQwen2Attention(QLlamaAttention):
+    """model/qQwenLayer.py:205-357: Qwen2's attention block built the reference's way.  Same calibration keys
+    ('layers.{i}.self_attn.{q,k,v,o}_proj.input', :227-249) and the same flow as the Llama block; what differs is
+    the model: q_proj / k_proj / v_proj carry a bias, which QLinearLayer adds behind the GEMM
+    (model/qLinearLayer.py:75-76), and the geometry (Qwen2.5-7B: hidden 3584, 28 query / 4 KV heads of 128)."""
+
+
+class QQwen2MLP(QLlamaMLP):
+    """model/qQwenLayer.py:360-425: keys 'layers.{i}.mlp.{gate,up,down}_proj.input' (:374-391).  The down
+    projection's input is 18944 wide in Qwen2.5-7B: the fused SwiGLU -> quantize pass and the quantizers take
+    rows of up to 32736 channels (the reference has dedicated kernels for exactly this width,
+    kernels/src/reorder.cu:380-555, dispatch kernels/src/bindings.cpp:141-160)."""
+
+
+class QQwen2DecoderLayer(QLlamaDecoderLayer):
+    """model/qQwenLayer.py:88-176: the decoder layer from its own linears (q / k / v with bias), norm weights and
+    the two calibration dicts."""
+
+    attention_class = QQwen2Attention
+    mlp_class = QQwen2MLP
+
+
+MOE_KEY = "layers.{}.{}.{}.{}.{}.{}"     # model/qMixtralLayer.py:488: layer, 'block_sparse_moe', 'experts', expert, projection, 'input'
+
+
+def _calibrated_expert(select_nums, reorder_index, layer_idx, moe_idx, proj, device):
+    key = MOE_KEY.format(layer_idx, "block_sparse_moe", "experts", moe_idx, proj, "input")
+    if key not in select_nums or key not in reorder_index:
+        raise KeyError(f"calibration files hold no entry {key}")
+    return int(select_nums[key]), reorder_index[key].to(device=device, dtype=torch.int16).contiguous()
+
+
+class QMixtralAttention(QLlamaAttention):
+    """model/qMixtralLayer.py:214-386: the four-part keys 'layers.{i}.self_attn.{q,k,v,o}_proj.input' (:246-272)
+    and the flow of the Llama block."""
+
+
+class QMixtralBlockSparseTop2MLP(nn.Module):
+    """model/qMixtralLayer.py:474-543 with the reference's constructor arguments: one expert's w1 / w3 / w2 and the
+    calibration dicts keyed 'layers.{i}.block_sparse_moe.experts.{e}.w{1,2,3}.input' (:488-508).  w1 and w3 stay
+    separate QLinearLayers with their own NVFP4 tensor scales, so the weight codes are the reference's; both read
+    the input quantized with w1's entry (:530), so w3's entry has to agree with it."""
+
+    def __init__(self, w1: nn.Linear, w3: nn.Linear, w2: nn.Linear, select_nums, reorder_index, layer_idx, moe_idx,
+                 quant_type="NVFP4"):
+        super().__init__()
+        dev = w1.weight.device
+        self.ffn_dim, self.hidden_dim = w1.out_features, w1.in_features
+        sel1, idx1 = _calibrated_expert(select_nums, reorder_index, layer_idx, moe_idx, "w1", dev)
+        sel3, idx3 = _calibrated_expert(select_nums, reorder_index, layer_idx, moe_idx, "w3", dev)
+        sel2, idx2 = _calibrated_expert(select_nums, reorder_index, layer_idx, moe_idx, "w2", dev)
+        if sel3 != sel1 or not torch.equal(idx3, idx1):
+            raise ValueError("w3 reads w1's quantized input: its select_num and reorder_index must equal w1's")
+        self.w1 = QLinearLayer(w1, sel1, idx1, quant_type=quant_type)
+        self.w3 = QLinearLayer(w3, sel3, idx3, quant_type=quant_type)
+        self.w2 = QLinearLayer(w2, sel2, idx2, quant_type=quant_type)
+        self.register_buffer("w1_reorder_index", idx1)
+        self.register_buffer("w2_reorder_index", idx2)
+        self.quant_type = quant_type
+
+    @torch.no_grad()
+    def forward(self, x):
+        """x bf16 [tokens of this expert, hidden] (model/qMixtralLayer.py:523-543)"""
+        xq = quantize_tokens(x, self.w1_reorder_index, self.w1.select_num, self.quant_type)
+        gate, up = self.w1(xq), self.w3(xq)
+        if self.ffn_dim <= 32736 and self.ffn_dim % 32 == 0:
+            nv = self.quant_type == "NVFP4"
+            r = agemm.swiglu_quantize_x(gate, up, self.w2_reorder_index, self.w2.select_num, fmt=self.quant_type,
+                                        global_scale="absmax" if nv else None)
+            return self.w2((r[0], r[1], r[2] if nv else 1.0, None, x.shape[0]))
+        return self.w2(quantize_tokens(F.silu(gate) * up, self.w2_reorder_index, self.w2.select_num, self.quant_type))
+
+
+class QMixtralSparseMoeBlock(MixtralSparseMoeBlock):
+    """model/qMixtralLayer.py:388-471 built the reference's way: the router, every expert's (w1, w3, w2) and the
+    calibration dicts; the experts become QMixtralBlockSparseTop2MLP (:419-420).  Routing, the expert-sorted rows
+    and the weighted sum are MixtralSparseMoeBlock's; the expert MLPs run as grouped launches over all experts
+    (w1 and w3 as two launches: each keeps the tensor scale of its own weight) when the experts agree on shapes
+    and select_nums, else as the reference's loop over experts."""
+
+    def __init__(self, gate: nn.Linear, experts, select_nums, reorder_index, i, quant_type="NVFP4", top_k=2,
+                 grouped=True):
+        nn.Module.__init__(self)
+        self.gate = gate
+        self.num_experts, self.top_k = len(experts), top_k
+        self.experts = nn.ModuleList([QMixtralBlockSparseTop2MLP(w1, w3, w2, select_nums, reorder_index, i, j, quant_type)
+                                      for j, (w1, w3, w2) in enumerate(experts)])
+        e0 = self.experts[0]
+        self.quant_type, self.ffn, self.interleaved = quant_type, e0.ffn_dim, False
+        same = all(ex.w1.W.shape == e0.w1.W.shape and ex.w2.W.shape == e0.w2.W.shape and
+                   ex.w1.select_num == e0.w1.select_num and ex.w2.select_num == e0.w2.select_num and
+                   ex.w1.bias is None and ex.w3.bias is None and ex.w2.bias is None for ex in self.experts)
+        kp1, kp2 = 2 * e0.w1.W.shape[1], 2 * e0.w2.W.shape[1]
+        self.grouped = bool(grouped) and same and kp1 % 128 == 0 and kp2 % 128 == 0 and min(kp1, kp2) >= 512 and \
+            e0.ffn_dim <= 32736 and e0.ffn_dim % 32 == 0 and e0.hidden_dim <= 32736
+        if self.grouped:
+            for name in ("w1", "w3", "w2"):
+                W = torch.stack([getattr(ex, name).W for ex in self.experts])
+                SF = torch.cat([getattr(ex, name).scale_w for ex in self.experts])
+                sc = torch.stack([getattr(ex, name).scale.reshape(()) for ex in self.experts]).to(torch.float32)
+                self.register_buffer(f"{name}_W", W)
+                self.register_buffer(f"{name}_scale_w", SF)
+                self.register_buffer(f"{name}_scale", sc)
+                per = SF.numel() // self.num_experts
+                for j, ex in enumerate(self.experts):        # the experts keep views, not copies
+                    lin = getattr(ex, name)
+                    lin.W, lin.scale_w, lin.scale = W[j], SF[j * per:(j + 1) * per], sc[j]
+            self.register_buffer("w1_reorder_index", torch.stack([ex.w1_reorder_index for ex in self.experts]))
+            self.register_buffer("w2_reorder_index", torch.stack([ex.w2_reorder_index for ex in self.experts]))
+            self.register_buffer("_expert_ids", torch.arange(self.num_experts, device=W.device))
+
+    def _experts_grouped(self, xs, seg):
+        e0, qt = self.experts[0], self.quant_type
+        nv = qt == "NVFP4"
+        gs = agemm.grouped_tensor_scale(xs, seg, NVFP4_RANGE) if nv else None
+        q, sf = agemm.grouped_reorder_quantize_x(xs, seg, self.w1_reorder_index, e0.w1.select_num, fmt=qt, global_scales=gs)
+        gate = agemm.grouped_matmul(q, self.w1_W, sf, self.w1_scale_w, seg, gs, self.w1_scale if nv else None, fmt=qt)
+        up = agemm.grouped_matmul(q, self.w3_W, sf, self.w3_scale_w, seg, gs, self.w3_scale if nv else None, fmt=qt)
+        if nv:
+            q2, sf2, gs2 = agemm.grouped_swiglu_quantize_x(gate, up, seg, self.w2_reorder_index, e0.w2.select_num, fmt=qt,
+                                                           global_scales="absmax")
+        else:
+            q2, sf2 = agemm.grouped_swiglu_quantize_x(gate, up, seg, self.w2_reorder_index, e0.w2.select_num, fmt=qt)
+            gs2 = None
+        return agemm.grouped_matmul(q2, self.w2_W, sf2, self.w2_scale_w, seg, gs2, self.w2_scale if nv else None, fmt=qt)
 
 
 class GraphedDecodeStep:

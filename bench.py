@@ -518,6 +518,25 @@ def main():
         name = {"x_unit": "reorder_quantize_x (tensor scale 1)", "x_scaled": "reorder_quantize_x (tensor scale max|x|/2688 on the device)"}[kind]
         quant.append({"op": name, "fmt": fmt, "select_num": S, "M": M_TOKENS, "us": round(ms * 1e3, 2),
                       "GB/s": round(b / ms / 1e6, 1), "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)})
+    # long rows: the down projection's input at Llama-3-8B width (14336) and at the reference's widest dedicated
+    # shape (28672, kernels/src/down.cu:71-233), 4096 rows each, tensor scale 1; rate per byte side by side
+    if not args.no_quantize_table:
+        for K in (14336, 28672):
+            nb = max(2, int(7e8 // (M_TOKENS * K * 2)))
+            xw = [recipes.activations(M_TOKENS, K, seed=20 + i).cuda() for i in range(2)]
+            xw += [xw[i % 2].roll(i, 0) for i in range(2, nb)]
+            iw = recipes.reorder_index(xw[0].cpu()).cuda()
+            for fmt in ("NVFP4", "MXFP4"):
+                q = torch.empty(L.arcq_codes_bytes(M_TOKENS, K, SELECT), dtype=torch.uint8, device="cuda")
+                sf = torch.empty(L.arcq_scales_bytes(M_TOKENS, K, SELECT, fid[fmt]), dtype=torch.uint8, device="cuda")
+                fn = lambda i, fmt=fmt, q=q, sf=sf, K=K: L.arcq_reorder_quantize_x(
+                    xw[i % nb].data_ptr(), M_TOKENS, K, iw.data_ptr(), SELECT, fid[fmt], 1.0, None, q.data_ptr(), sf.data_ptr(), stream)
+                ms = time_quant(fn, M_TOKENS, 50)
+                b = quant_bytes(M_TOKENS, K, SELECT, fmt, False)
+                quant.append({"op": "reorder_quantize_x (tensor scale 1)", "fmt": fmt, "select_num": SELECT, "M": M_TOKENS, "K": K,
+                              "us": round(ms * 1e3, 2), "GB/s": round(b / ms / 1e6, 1), "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)})
+            del xw
+            torch.cuda.empty_cache()
     out["quantize"] = quant
     del xs[1:], outs[1:], sdst[1:]
     torch.cuda.empty_cache()

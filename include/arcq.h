@@ -133,7 +133,7 @@ int arcq_rmsnorm_quantize_x(const void *x, const void *gamma, float eps, int M, 
  * fusion but does not ship it (benchmarks/modeling_arc.py:112, commented activate_quantize_x).
  *   gate, up  bf16 rows of K elements with a common row stride `ld` (elements, multiple of 8): for a
  *             fused gate_up projection output [M, 2K] pass up = gate + K and ld = 2K
- *   K         multiple of 32, 32 <= K <= 16384
+ *   K         multiple of 32, 32 <= K <= 32736
  * arcq_swiglu_absmax computes max |t| over the tensor (numerator of the NVFP4 tensor scale,
  * model/qLlamaLayer.py:74) into *d_absmax, which the caller has set to 0; nothing synchronises.
  */
@@ -220,7 +220,7 @@ size_t arcq_matmul_scratch_bytes(int M, int N, int Kp, int fmt);
  * Nothing is read back to the host.  Codes and scale bytes of a row are those arcq_reorder_quantize_x /
  * arcq_swiglu_quantize_x write for that row with its expert's index and scale.
  * arcq_grouped_tensor_scale writes the n_seg scales (1 for an expert without rows or with only zeros);
- * `up` as for arcq_tensor_scale.  K <= 16384 for the quantizers.
+ * `up` as for arcq_tensor_scale.  K <= 32736 for the quantizers.
  */
 int arcq_grouped_reorder_quantize_x(const void *x, int M, int K, const int *seg_offsets, int n_seg,
                                     const int16_t *reorder_index, int select_num, int fmt, const float *d_global_scales,

@@ -45,7 +45,7 @@ COUNTS = [[5, 0, 17, 1, 300, 0, 64, 9], [40], [0, 0, 3], [130, 131, 2, 700]]
 
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("counts", COUNTS)
-@pytest.mark.parametrize("K,S", [(4096, 128), (512, 512), (1024, 0)])
+@pytest.mark.parametrize("K,S", [(4096, 128), (512, 512), (1024, 0), (18944, 256)])
 def test_grouped_quantize_matches_per_expert_oracle(agemm, oracle, fmt, counts, K, S):
     T, E = sum(counts), len(counts)
     x = recipes.activations(T, K, seed=7000 + T + K, outlier_frac=0.01, outlier_gain=40.0)
@@ -75,9 +75,9 @@ def test_grouped_quantize_matches_per_expert_oracle(agemm, oracle, fmt, counts, 
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-@pytest.mark.parametrize("counts", [[5, 0, 17, 1, 300, 0, 64, 9], [700, 3]])
-def test_grouped_swiglu_matches_ungrouped(agemm, fmt, counts):
-    T, E, F, S = sum(counts), len(counts), 1024, 128
+@pytest.mark.parametrize("counts,F", [([5, 0, 17, 1, 300, 0, 64, 9], 1024), ([700, 3], 1024), ([40, 0, 290], 18944)])
+def test_grouped_swiglu_matches_ungrouped(agemm, fmt, counts, F):
+    T, E, S = sum(counts), len(counts), 128
     g = torch.Generator().manual_seed(T)
     gu = (torch.randn(T, 2 * F, generator=g) * 2.0).to(torch.bfloat16).cuda()
     seg = segments(counts)

@@ -447,3 +447,180 @@ def test_decoder_layer_from_calibration_files(layers, fq, oracle, fmt, tmp_path)
     fused = layers.QLlamaDecoderLayer(lin, (g1.cuda(), g2.cuda()), eps, nh, nkv, sn, ri, li, quant_type=fmt,
                                       fuse_norm=True)
     assert rel_fro(fused(x.cuda()), y) < 0.1
+
+
+def c_ref_linear(oracle, x, w, idx, S, fmt, bias=None):
+    """one ARC linear of the fake-quant flow through the C oracle (model/quantize.py:287-343, model/qLinearLayer.py:65-81):
+    activations with the callers' tensor scale max|x| / 2688, weights with the signed max / 2688, fp32 product of the
+    dequantized operands, bf16 output, bias behind it"""
+    import numpy as np
+    gx = float(x.abs().max().float() / torch.tensor(2688.0)) if fmt == "NVFP4" else 1.0
+    gw = recipes.tensor_scale(w, fmt)
+    a = oracle.quantize_x(x, idx, S, fmt, gx, want_dq=True)["dq"]
+    b = oracle.quantize_w(w, idx, S, fmt, gw, want_dq=True)["dq"]
+    y = (torch.from_numpy(a) @ torch.from_numpy(b).T * np.float32(gx * gw)).to(torch.bfloat16)
+    return y if bias is None else y + bias
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_qwen_decoder_layer_at_its_geometry(layers, fq, oracle, fmt, tmp_path):
+    """Qwen2.5-7B's decoder layer (model/qQwenLayer.py:88-176, 227-249, 374-391): hidden 3584, 28 query and 4 KV
+    heads of 128, q / k / v with bias, intermediate 18944 -- the down projection's input is wider than 16384
+    channels and takes the four-units-per-thread quantizers.  Built from calibration files; 48 tokens against the
+    fake-quant flow on the CPU (C oracle quantizers, fp32 products)."""
+    from arcquant_amd import calibration as cal
+    hidden, inter, nh, nkv, eps, li = 3584, 18944, 28, 4, 1e-6, 0
+    bsz, q_len, d = 2, 24, 128
+    g = torch.Generator().manual_seed(71)
+    shapes = {"q_proj": (nh * d, hidden), "k_proj": (nkv * d, hidden), "v_proj": (nkv * d, hidden),
+              "o_proj": (hidden, hidden), "gate_proj": (inter, hidden), "up_proj": (inter, hidden),
+              "down_proj": (hidden, inter)}
+    W = {k: (torch.randn(*s, generator=g) * 0.02).to(torch.bfloat16) for k, s in shapes.items()}
+    B = {k: (torch.randn(shapes[k][0], generator=g) * 0.2).to(torch.bfloat16) for k in ("q_proj", "k_proj", "v_proj")}
+    g1 = (torch.rand(hidden, generator=g) + 0.5).to(torch.bfloat16)
+    g2 = (torch.rand(hidden, generator=g) + 0.5).to(torch.bfloat16)
+    x = torch.randn(bsz, q_len, hidden, generator=g)
+    x[..., 11] *= 20.0
+    x = x.to(torch.bfloat16)
+    stat = {"attn": torch.rand(hidden, generator=g), "o": torch.rand(hidden, generator=g),
+            "mlp": torch.rand(hidden, generator=g), "down": torch.rand(inter, generator=g)}
+    block_of = {"q_proj": ("self_attn", "attn", 128), "k_proj": ("self_attn", "attn", 128), "v_proj": ("self_attn", "attn", 128),
+                "o_proj": ("self_attn", "o", 128), "gate_proj": ("mlp", "mlp", 128), "up_proj": ("mlp", "mlp", 128),
+                "down_proj": ("mlp", "down", 256)}
+    ri, sn = {}, {}
+    for proj, (block, st, sel) in block_of.items():
+        key = cal.NAME_TEMPLATE.format(li, block, proj)
+        ri[key] = cal.reorder_index_from_stat(stat[st])
+        sn[key] = sel
+    cal.save_reorder_index(tmp_path / "reorder_index.pt", ri)
+    cal.save_select_num(tmp_path / "select_num.pt", sn)
+    ri, sn = cal.load_reorder_index(tmp_path / "reorder_index.pt"), cal.load_select_num(tmp_path / "select_num.pt")
+    lin = {}
+    for k, (n_out, n_in) in shapes.items():
+        lin[k] = nn.Linear(n_in, n_out, bias=k in B, device="cuda", dtype=torch.bfloat16)
+        lin[k].weight.data.copy_(W[k])
+        if k in B:
+            lin[k].bias.data.copy_(B[k])
+    print(f"Qwen2.5-7B decoder layer {fmt}", flush=True)
+    layer = layers.QQwen2DecoderLayer(lin, (g1.cuda(), g2.cuda()), eps, nh, nkv, sn, ri, li, quant_type=fmt)
+    assert isinstance(layer.self_attn, layers.QQwen2Attention) and isinstance(layer.mlp, layers.QQwen2MLP)
+    assert layer.self_attn.q_proj.bias is not None and layer.self_attn.o_proj.bias is None
+    # the wide projection's weights: codes and scale bytes against the oracle
+    idx_d = ri[cal.NAME_TEMPLATE.format(li, "mlp", "down_proj")].to(torch.int16)
+    want = oracle.quantize_w(W["down_proj"], idx_d, 256, fmt, recipes.tensor_scale(W["down_proj"], fmt))
+    assert (layer.mlp.down_proj.W.cpu().numpy() == want["codes"]).all()
+    assert (layer.mlp.down_proj.scale_w.cpu().numpy().reshape(want["scales"].shape) == want["scales"]).all()
+
+    y = layer(x.cuda())
+    torch.cuda.synchronize()
+    assert y.shape == x.shape
+
+    def lin_ref(t, proj):
+        block, st, sel = block_of[proj]
+        idx = ri[cal.NAME_TEMPLATE.format(li, block, proj)].to(torch.int16)
+        return c_ref_linear(oracle, t, W[proj], idx, sel, fmt, B.get(proj))
+
+    x2 = x.view(-1, hidden)
+    n1 = fq.hf_rmsnorm(x2, g1, eps)
+    qkv = torch.cat([lin_ref(n1, p) for p in ("q_proj", "k_proj", "v_proj")], dim=1)
+    q = qkv[:, :nh * d].view(bsz, q_len, nh, d).transpose(1, 2)
+    k = qkv[:, nh * d:(nh + nkv) * d].view(bsz, q_len, nkv, d).transpose(1, 2)
+    v = qkv[:, (nh + nkv) * d:].view(bsz, q_len, nkv, d).transpose(1, 2)
+    q, k = layers.rotary_pos_emb(q, k, 0)
+    k, v = k.repeat_interleave(nh // nkv, 1), v.repeat_interleave(nh // nkv, 1)
+    o = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True).to(torch.bfloat16)
+    h = x2 + lin_ref(o.transpose(1, 2).reshape(bsz * q_len, hidden), "o_proj")
+    n2 = fq.hf_rmsnorm(h, g2, eps)
+    t = F.silu(lin_ref(n2, "gate_proj")) * lin_ref(n2, "up_proj")
+    want = h + lin_ref(t, "down_proj")
+    # Block by block, each fed the reference's input: a 4-bit layer turns a 1 % difference of its input (here the
+    # bf16 attention against the fp32 one, then requantized) into a different set of codes, i.e. into its own
+    # quantization noise, so the end-to-end figure says little about the operators
+    a, m = layer.self_attn, layer.mlp
+    xc = x.cuda()
+    n1g = layer.input_layernorm(xc)
+    assert torch.equal(n1g.view(-1, hidden).cpu(), n1)
+    tq = layers.quantize_tokens(n1g, a.q_reorder_index, a.q_proj.select_num, fmt)
+    assert rel_fro(a.qkv_proj(tq).view(-1, qkv.shape[1]), qkv) < 5e-3          # three projections with their biases
+    assert rel_fro(a(tq, None, 0, li, residual=xc).view(-1, hidden), h) < 2e-2   # bf16 SDPA, o_proj on its output
+    hc = h.cuda().view(bsz, q_len, hidden)
+    tq2 = layers.quantize_tokens(layer.post_attention_layernorm(hc), m.up_reorder_index, m.up_proj.select_num, fmt)
+    assert rel_fro(m(tq2, residual=hc).view(-1, hidden), want) < 5e-3          # gate / up, SwiGLU over 18944 channels, down
+    assert rel_fro(y.view(-1, hidden), want) < 0.25                            # the whole layer: within quantization noise
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("grouped", [True, False])
+def test_mixtral_block_from_calibration_files(layers, oracle, fmt, grouped, tmp_path):
+    """The reference's way of building the MoE block (model/qMixtralLayer.py:400-420, 488-508): calibration dicts
+    keyed 'layers.{i}.block_sparse_moe.experts.{e}.w{1,2,3}.input' written and read in its file format, every
+    expert's w1 / w3 / w2 a QLinearLayer of its own (weight codes and scale bytes bit for bit the oracle's, each
+    with the tensor scale of its own weight); the block's output against the reference's loop over experts with
+    the C oracle's quantizers on the CPU (model/qMixtralLayer.py:441-471, 523-543)."""
+    from arcquant_amd import calibration as cal
+    hidden, ffn, E, li, tokens = 384, 512, 4, 5, 96
+    g = torch.Generator().manual_seed(81)
+    ri, sn, Wt = {}, {}, []
+    for e in range(E):
+        i_in = cal.reorder_index_from_stat(torch.rand(hidden, generator=g))
+        i_w2 = cal.reorder_index_from_stat(torch.rand(ffn, generator=g))
+        for proj, idx, sel in (("w1", i_in, 128), ("w3", i_in, 128), ("w2", i_w2, 128)):
+            ri[cal.MOE_NAME_TEMPLATE.format(li, e, proj)] = idx
+            sn[cal.MOE_NAME_TEMPLATE.format(li, e, proj)] = sel
+        Wt.append({"w1": (torch.randn(ffn, hidden, generator=g) * 0.05 * (1 + e)).to(torch.bfloat16),
+                   "w3": (torch.randn(ffn, hidden, generator=g) * 0.02).to(torch.bfloat16),
+                   "w2": (torch.randn(hidden, ffn, generator=g) * 0.03).to(torch.bfloat16)})
+    cal.save_reorder_index(tmp_path / "ri.pt", ri)
+    cal.save_select_num(tmp_path / "sn.pt", sn)
+    ri, sn = cal.load_reorder_index(tmp_path / "ri.pt"), cal.load_select_num(tmp_path / "sn.pt")
+
+    def linear(w):
+        m = nn.Linear(w.shape[1], w.shape[0], bias=False, device="cuda", dtype=torch.bfloat16)
+        m.weight.data.copy_(w)
+        return m
+    gate = nn.Linear(hidden, E, bias=False, device="cuda", dtype=torch.bfloat16)
+    experts = [(linear(w["w1"]), linear(w["w3"]), linear(w["w2"])) for w in Wt]
+    print(f"calibrated mixtral block {fmt} grouped={grouped}", flush=True)
+    block = layers.QMixtralSparseMoeBlock(gate, experts, sn, ri, li, quant_type=fmt, grouped=grouped)
+    assert block.grouped == grouped
+    with pytest.raises(KeyError):
+        layers.QMixtralSparseMoeBlock(gate, experts, sn, ri, li + 1, quant_type=fmt)
+    for e, ex in enumerate(block.experts):
+        for proj in ("w1", "w3", "w2"):
+            key = cal.MOE_NAME_TEMPLATE.format(li, e, proj)
+            gw = recipes.tensor_scale(Wt[e][proj], fmt)
+            want = oracle.quantize_w(Wt[e][proj], ri[key].to(torch.int16), sn[key], fmt, gw)
+            m = getattr(ex, proj)
+            assert (m.W.cpu().numpy() == want["codes"]).all(), (e, proj)
+            assert (m.scale_w.cpu().numpy().reshape(want["scales"].shape) == want["scales"]).all(), (e, proj)
+            assert float(m.scale) == pytest.approx(gw, rel=1e-7)
+    if fmt == "NVFP4":
+        assert float(block.experts[1].w1.scale) != float(block.experts[1].w3.scale)
+
+    x = torch.randn(1, tokens, hidden, generator=g).to(torch.bfloat16)
+    logits = torch.randn(tokens, E, generator=g)
+    logits[:, 2] -= 100.0                                   # an expert that receives no token
+    y, _ = block(x.cuda(), router_logits=logits.cuda())
+    torch.cuda.synchronize()
+
+    w = F.softmax(logits, dim=1, dtype=torch.float)
+    w, sel = torch.topk(w, 2, dim=-1)
+    w = (w / w.sum(dim=-1, keepdim=True)).to(torch.bfloat16)
+    want = torch.zeros(tokens, hidden, dtype=torch.bfloat16)
+    x2 = x.view(tokens, hidden)
+    for e in range(E):
+        slot, top_x = torch.where((sel == e).T)
+        if top_x.numel() == 0:
+            continue
+        k1, k2 = cal.MOE_NAME_TEMPLATE.format(li, e, "w1"), cal.MOE_NAME_TEMPLATE.format(li, e, "w2")
+        cur = x2[top_x]
+        h1 = c_ref_linear(oracle, cur, Wt[e]["w1"], ri[k1].to(torch.int16), sn[k1], fmt)
+        h3 = c_ref_linear(oracle, cur, Wt[e]["w3"], ri[k1].to(torch.int16), sn[k1], fmt)
+        out = c_ref_linear(oracle, F.silu(h1) * h3, Wt[e]["w2"], ri[k2].to(torch.int16), sn[k2], fmt)
+        want.index_add_(0, top_x, out * w[top_x, slot, None])
+    assert rel_fro(y.view(tokens, hidden), want) < 2e-2
+    # w3's entry must agree with w1's: both projections read one quantized input (model/qMixtralLayer.py:530-535)
+    bad = dict(ri)
+    bad[cal.MOE_NAME_TEMPLATE.format(li, 0, "w3")] = torch.flip(ri[cal.MOE_NAME_TEMPLATE.format(li, 0, "w3")], [0])
+    with pytest.raises(ValueError):
+        layers.QMixtralSparseMoeBlock(gate, experts, sn, bad, li, quant_type=fmt)

@@ -284,3 +284,28 @@ def test_quantizers_random_shapes(agemm, oracle, seed):
             q, sf = agemm.rmsnorm_quantize_x(dev(x), dev(gamma), 1e-5, dev(idx), S, fmt=fmt, global_scale=gs)
         compare(f"{mode} {fmt} M={M} K={K} S={S}", q, sf, want)
         done += 1
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("M,K,S", [(300, 18944, 256), (257, 27648, 512), (256, 28672, 128), (40, 32736, 64), (3, 16416, 0),
+                                   (700, 28672, 1024)])
+def test_rows_of_more_than_16384_channels(agemm, oracle, fmt, M, K, S):
+    """The reference's dedicated wide shapes (K = 18944: kernels/src/reorder.cu:380-555; 27648 and 28672:
+    kernels/src/down.cu:71-233; dispatch kernels/src/bindings.cpp:141-160) and the longest row an int16 index
+    allows: four units per thread.  Activations with tensor scale 1 and with the NVFP4 tensor scale (host value
+    and device scalar), weights; every row against the oracle."""
+    x = recipes.activations(M, K, seed=6000 + M + K)
+    x[M // 2] = 0
+    idx = recipes.reorder_index(x)
+    print(f"wide rows {fmt} M={M} K={K} S={S}", flush=True)
+    for gs in ((1.0, recipes.nvfp4_tensor_scale(x)) if fmt == "NVFP4" else (1.0, 0.5)):
+        want = oracle.quantize_x(x, idx, S, fmt, gs)
+        q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), S, fmt=fmt, global_scale=gs)
+        compare(f"x, tensor scale {gs}", q, sf, want)
+        q, sf = agemm.reorder_quantize_x(dev(x), dev(idx), S, fmt=fmt, global_scale=torch.tensor(gs, dtype=torch.float32).cuda())
+        compare(f"x, tensor scale {gs} on the device", q, sf, want)
+    w = recipes.weights(M, K, seed=6001 + M)
+    gw = recipes.tensor_scale(w, fmt)
+    want = oracle.quantize_w(w, idx, S, fmt, gw)
+    q, sf = agemm.reorder_quantize_w(dev(w), dev(idx), S, fmt=fmt, global_scale=gw)
+    compare("w", q, sf, want)

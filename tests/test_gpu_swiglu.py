@@ -34,7 +34,8 @@ def inputs(M, K, seed):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
-@pytest.mark.parametrize("M,K,S", [(1, 512, 64), (33, 1024, 128), (16, 14336, 256), (130, 2048, 0)])
+@pytest.mark.parametrize("M,K,S", [(1, 512, 64), (33, 1024, 128), (16, 14336, 256), (130, 2048, 0), (70, 18944, 256),
+                                   (33, 28672, 512)])
 def test_fused_equals_unfused_on_gpu(agemm, oracle, fmt, M, K, S):
     gu = inputs(M, K, seed=70 + M)
     gud = gu.cuda()
