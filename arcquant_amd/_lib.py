@@ -91,16 +91,34 @@ def lib() -> ctypes.CDLL:
         getattr(L, name).restype = i
     L.arcq_check_index.argtypes = [vp, i, vp]
     L.arcq_dequantize.argtypes = [vp, vp, i, i, i, vp, vp]
-    L.arcq_stream_probe.argtypes = [vp, vp, sz, sz, vp]
-    L.arcq_stream_probe_variant.argtypes = [vp, vp, sz, sz, i, vp]
-    L.arcq_stream_probe_variant.restype = i
-    L.arcq_stream_probe_variants.restype = i
     for name in ("arcq_reorder_quantize_x", "arcq_reorder_quantize_w", "arcq_rmsnorm_quantize_x", "arcq_matmul",
-                 "arcq_check_index", "arcq_dequantize", "arcq_stream_probe", "arcq_swiglu_quantize_x", "arcq_swiglu_absmax",
+                 "arcq_check_index", "arcq_dequantize", "arcq_swiglu_quantize_x", "arcq_swiglu_absmax",
                  "arcq_kv_append_i4", "arcq_kv_store_i4", "arcq_kv_decode_i4"):
         getattr(L, name).restype = i
     _lib = L
     return L
+
+
+PROBE_LIB_PATH = os.path.join(_HERE, "csrc", "libarcq_probe.so")
+_probe = None
+
+
+def probe_lib() -> ctypes.CDLL:
+    """libarcq_probe.so (include/arcq_probe.h): plain copy kernels, for measurement only -- bench.py's streaming
+    ceiling and the calibration of the rocprofv3 traffic counters.  No operator loads it."""
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_LIB_PATH):
+            raise RuntimeError(f"{PROBE_LIB_PATH} is missing: build it with `python -m arcquant_amd.build`")
+        P = ctypes.CDLL(PROBE_LIB_PATH)
+        vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+        P.arcq_stream_probe.argtypes = [vp, vp, sz, sz, vp]
+        P.arcq_stream_probe.restype = i
+        P.arcq_stream_probe_variant.argtypes = [vp, vp, sz, sz, i, vp]
+        P.arcq_stream_probe_variant.restype = i
+        P.arcq_stream_probe_variants.restype = i
+        _probe = P
+    return _probe
 
 
 def check(status: int, where: str) -> None:

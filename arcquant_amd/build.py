@@ -17,6 +17,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 HIP_SOURCES = ["arcq_common.hip", "arcq_quantize.hip", "arcq_gemm.hip", "arcq_kvcache.hip", "arcq_moe.hip"]
 HIP_LIB = os.path.join(CSRC, "libarcq_hip.so")
+# measurement only (plain copy kernels for bench.py and the counter calibration): its own library, so that the
+# product library holds operators only
+PROBE_LIB = os.path.join(CSRC, "libarcq_probe.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -54,8 +57,18 @@ def build_hip(force: bool = False, verbose: bool = False) -> str:
     return HIP_LIB
 
 
+def build_probe(force: bool = False, verbose: bool = False) -> str:
+    src = os.path.join(CSRC, "arcq_probe.hip")
+    if force or _stale(PROBE_LIB, [src, os.path.join(HERE, "..", "include", "arcq_probe.h")]):
+        cmd = [_hipcc(), *HIPCC_FLAGS, "-o", PROBE_LIB, src]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
+    return PROBE_LIB
+
+
 def build_all(force: bool = False, verbose: bool = False):
-    return (build_hip(force, verbose),)
+    return (build_hip(force, verbose), build_probe(force, verbose))
 
 
 if __name__ == "__main__":

@@ -447,9 +447,10 @@ def main():
     b_out = ((bytes_per_launch - b_in) // 16) * 16
     sdst = [torch.empty(b_out, dtype=torch.uint8, device="cuda") for _ in range(nbuf)]
     probes = {}
-    for variant in range(L.arcq_stream_probe_variants()):
+    P = _lib.probe_lib()                                   # measurement-only library of plain copy kernels
+    for variant in range(P.arcq_stream_probe_variants()):
         def probe(i, variant=variant):
-            L.arcq_stream_probe_variant(xs[i % nbuf].data_ptr(), sdst[i % nbuf].data_ptr(), b_in, b_out, variant, stream)
+            P.arcq_stream_probe_variant(xs[i % nbuf].data_ptr(), sdst[i % nbuf].data_ptr(), b_in, b_out, variant, stream)
         for i in range(10):
             probe(i)
         probes[variant] = loop_time_ms(probe, 100, torch)

@@ -386,25 +386,6 @@ int arcq_check_index(const int16_t *reorder_index, int K, void *stream);
  */
 int arcq_dequantize(const void *codes, const void *scales, int rows, int Kp, int fmt, float *out, void *stream);
 
-/*
- * Measurement helper (no counterpart in the reference): a plain streaming kernel that reads
- * bytes_in from src and writes the first bytes_out of them to dst (multiples of 16, bytes_out <=
- * bytes_in).  bench.py times it with the quantizers' read:write ratio as the achievable HBM
- * ceiling of the box, and the rocprof FETCH_SIZE / WRITE_SIZE readings are calibrated on it.
- */
-int arcq_stream_probe(const void *src, void *dst, size_t bytes_in, size_t bytes_out, void *stream);
-
-/*
- * The same copy with other launch shapes (no counterpart in the reference): variant 0 is
- * arcq_stream_probe (one 16-byte load in flight per thread); the others keep 2, 4 or 8 independent loads
- * in flight per thread, use non-temporal loads and stores, run as many workgroups as the chip holds or
- * exactly one round of threads, or go through LDS-direct loads.  bench.py times all of them on the
- * headline launch's bytes and reports the fastest as the streaming ceiling of the box.
- * arcq_stream_probe_variants() is their number; an unknown variant is ARCQ_ERR_SHAPE.
- */
-int arcq_stream_probe_variant(const void *src, void *dst, size_t bytes_in, size_t bytes_out, int variant, void *stream);
-int arcq_stream_probe_variants(void);
-
 #ifdef __cplusplus
 }
 #endif

@@ -11,8 +11,8 @@ from arcquant_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "arcq.h")).read()
+def declared_symbols(header="arcq.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(arcq_[a-z0-9_]+)\s*\(", text)))
 
@@ -109,8 +109,9 @@ def test_grouped_entry_points_reject_bad_arguments():
     assert mr(ok, 0, 16, 4, 5, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None) == 2                # top_k > experts
     assert mr(None, 0, 16, 8, 2, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None) == 1
     assert mr(ok, 0, 4096, 8, 2, ok, ok, ok, ok, ok, ok, ok, 16, None) == 7                   # workspace too small
-    assert L.arcq_stream_probe_variants() >= 2
-    assert L.arcq_stream_probe_variant(ok, ok, 1024, 512, 99, None) == 2
+    P = _lib.probe_lib()                 # the measurement-only library (include/arcq_probe.h)
+    assert P.arcq_stream_probe_variants() >= 2
+    assert P.arcq_stream_probe_variant(ok, ok, 1024, 512, 99, None) == 2
 
 
 def test_decode_batches_fit_the_no_alloc_array():
@@ -129,3 +130,12 @@ def test_decode_batches_fit_the_no_alloc_array():
 
 def test_release_stream_without_buffers_needs_no_gpu_work():
     assert hasattr(_lib.lib(), "arcq_release_stream")
+
+
+def test_probe_library_is_separate_from_the_product_library():
+    """the copy kernels used for measurement live in their own library with their own header"""
+    P, L = _lib.probe_lib(), _lib.lib()
+    names = declared_symbols("arcq_probe.h")
+    assert names == ["arcq_stream_probe", "arcq_stream_probe_variant", "arcq_stream_probe_variants"]
+    for n in names:
+        assert hasattr(P, n) and not hasattr(L, n)
