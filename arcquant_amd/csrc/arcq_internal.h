@@ -25,12 +25,12 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 // kept until the process ends, so that a captured graph may hold its address.  Work on one stream is
 // serialised, so two calls never share a buffer unless they share a stream.
 enum WorkspaceKind {
-  kWsTensorScale = 0,  // running maximum + arrival counter of arcq_tensor_scale (zeroed once)
+  kWsTensorScale = 0,  // (maximum, arrival counter) pairs of arcq_tensor_scale, one per 128-byte line (zeroed once)
   kWsSplitK = 1,       // fp32 partial tiles of the split-K GEMM
   kWsDecode = 2,       // partial softmax sums of the split decode attention
   kWsKinds = 3
 };
-constexpr size_t kWorkspaceBytes[kWsKinds] = {256, 32u << 20, 8u << 20};
+constexpr size_t kWorkspaceBytes[kWsKinds] = {2048, 32u << 20, 8u << 20};
 
 // The buffer of `kind` for (current device, stream).  Returns nullptr and sets *status when there is
 // none and none can be made: ARCQ_ERR_WORKSPACE while `stream` is capturing (an allocation there

@@ -149,7 +149,8 @@ ARCQ_HD float rcp_from_estimate(float s, float r0) {
 
 // Midpoint between grid magnitudes m and m+1 (m = 0..6): 0.25 0.75 1.25 1.75 2.5 3.5 5
 ARCQ_HD float e2m1_midpoint(uint32_t m) {
-  return m < 4u ? 0.25f + 0.5f * (float)m : (m == 4u ? 2.5f : (m == 5u ? 3.5f : 5.0f));
+  // as bits, without a branch: 0.25 and 0.75 are 0xc00000 apart, from 1.25 on the steps are 0x400000
+  return u2f(m < 2u ? 0x3e800000u + m * 0x00c00000u : 0x3f200000u + m * 0x00400000u);
 }
 
 // The reference's code for y/s when two conversions of approximate quotients just below and just

@@ -342,6 +342,42 @@ __device__ __forceinline__ uint2 encode_unit_two_sided(const float (&y)[16], flo
                     resolve_word(y[8], y[9], y[10], y[11], y[12], y[13], y[14], y[15], s, a1, b1));
 }
 
+// The same for a unit under a tensor scale g whose values y = x / g have not been formed: the two conversions start
+// from the raw bf16 x with R ~ 1 / (g * s) (R = RN(rg * r)); an element on which they differ gets its exact
+// y = RN(x / g) and goes through e2m1_resolve as above.  (tests/test_hostmath.py sweeps this against the reference's
+// code of RN(RN(x/g) / s) for every bf16 x, block scale, reciprocal within an ulp and tensor scale max / 2688.)
+__device__ __forceinline__ uint32_t resolve_word_x(float v0, float v1, float v2, float v3, float v4, float v5, float v6,
+                                                   float v7, float g, float rg, float s, uint32_t a, uint32_t b) {
+  uint32_t out = drop_negative_zeros(a);
+  uint32_t d = a ^ b;
+  while (d) {
+    const int nib = __builtin_ctz(d) >> 2;
+    const float a0 = (nib & 1) ? v1 : v0, a1 = (nib & 1) ? v3 : v2;
+    const float a2 = (nib & 1) ? v5 : v4, a3 = (nib & 1) ? v7 : v6;
+    const float b0 = (nib & 2) ? a1 : a0, b1 = (nib & 2) ? a3 : a2;
+    const float xi = (nib & 4) ? b1 : b0;
+    const uint32_t sh = 4u * (uint32_t)nib;
+    const uint32_t c = e2m1_resolve(div_bf16_by(xi, g, rg), s, (a >> sh) & 15u, (b >> sh) & 15u);
+    out = (out & ~(15u << sh)) | (c << sh);
+    d &= ~(15u << sh);
+  }
+  return out;
+}
+
+__device__ __forceinline__ uint2 encode_unit_two_sided_x(const float (&x)[16], float g, float rg, float s, float R) {
+  const float ra = R * 0x1.00001p+0f, rb = R * 0x1.ffffep-1f;
+  uint32_t a0 = 0u, a1 = 0u, b0 = 0u, b1 = 0u;
+#define ARCQ_ENC2(dst, rr, i, sel) \
+  dst = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(dst, x[i] * rr, x[i + 1] * rr, 1.0f, sel);
+  ARCQ_ENC2(a0, ra, 0, 0) ARCQ_ENC2(a0, ra, 2, 1) ARCQ_ENC2(a0, ra, 4, 2) ARCQ_ENC2(a0, ra, 6, 3)
+  ARCQ_ENC2(a1, ra, 8, 0) ARCQ_ENC2(a1, ra, 10, 1) ARCQ_ENC2(a1, ra, 12, 2) ARCQ_ENC2(a1, ra, 14, 3)
+  ARCQ_ENC2(b0, rb, 0, 0) ARCQ_ENC2(b0, rb, 2, 1) ARCQ_ENC2(b0, rb, 4, 2) ARCQ_ENC2(b0, rb, 6, 3)
+  ARCQ_ENC2(b1, rb, 8, 0) ARCQ_ENC2(b1, rb, 10, 1) ARCQ_ENC2(b1, rb, 12, 2) ARCQ_ENC2(b1, rb, 14, 3)
+#undef ARCQ_ENC2
+  return make_uint2(resolve_word_x(x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7], g, rg, s, a0, b0),
+                    resolve_word_x(x[8], x[9], x[10], x[11], x[12], x[13], x[14], x[15], g, rg, s, a1, b1));
+}
+
 // amax values for which the division-free arithmetic above is not trusted (results that
 // underflow or overflow on the way): everything but zero and the comfortable normal range
 __device__ __forceinline__ bool amax_needs_exact(float a) {
@@ -379,6 +415,23 @@ __device__ __forceinline__ void quantize_unit(const uint32_t (&yv)[16], bool act
 #pragma unroll
   for (int i = 0; i < 16; ++i) y[i] = u2f(yv[i]);
   if (SCALED) {
+    // A tensor scale that is not a power of two, and no lane of the wave has a residual to form (those need
+    // y = x / g itself): one division per unit.  RN(x / g) is monotone in |x|, so the block maximum of y is the
+    // quotient of the block maximum of x; the codes come straight from x (encode_unit_two_sided_x).
+    const bool wave_has_tail = MODE != MODE_W && __builtin_amdgcn_ballot_w64(tail) != 0ull;
+    if (!coarse && !wave_has_tail) {
+      float s;
+      const float amax = div_bf16_by(unit_amax3<FMT>(y), g, rg);
+      const float t = div6_any(amax);
+      sb = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t, &s) : ue8m0_scale(t, &s);
+      pk = encode_unit_two_sided_x(y, g, rg, s, rg * scale_rcp<FMT>(s));
+      bool redo = amax_needs_exact(amax) || g_odd;
+      if (FMT == ARCQ_FMT_MXFP4) redo = __shfl_xor((int)redo, 1) != 0 || redo;
+      if (redo && active) unit_exact<FMT, false>(yv, g, &pk, &sb, &pk2, &sb2);
+      pk2 = pk;
+      sb2 = sb;
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < 16; ++i) y[i] = div_bf16_by(y[i], g, rg);
   }
@@ -1019,36 +1072,51 @@ __global__ __launch_bounds__(256) void swiglu_absmax_kernel(const uint16_t *gate
 }
 
 // NVFP4 tensor scale of an activation tensor in one launch: max |x| / divisor (model/qLlamaLayer.py:74),
-// 1 for an all-zero tensor, as an fp32 scalar on the device.  SWIGLU: x = act_fn(gate) * up formed on the
-// fly.  Blocks meet through two words of a persistent workspace (running maximum as the bits of a
-// non-negative float, arrival counter): the last block to arrive divides, writes the scale and puts
-// both words back to zero.  Only device-scope atomics touch the two words, and a block's arrival is
-// issued after its maximum has returned, so the last block reads the maximum of all of them.
+// 1 for an all-zero tensor, as an fp32 scalar on the device.  SWIGLU: x = act_fn(gate) * up formed on the fly.
+//
+// A read-only stream: at most one workgroup of 512 or 1024 threads per CU, every thread with eight (SwiGLU: four per
+// operand) independent 16-byte loads in flight per trip.  The workgroups then meet through a persistent
+// workspace touched only by device-scope atomics.  Atomics on one word are served one after the other (10-30 ns
+// each: with a thousand workgroups arriving on one counter the launch spent 30 us there), so they meet in two
+// levels: a workgroup arrives at the (maximum, counter) pair of its group -- blockIdx mod kScaleGroups, each pair
+// on a cache line of its own -- and the
+// last arrival of a group arrives at the top counter; the last arrival there reads the groups' maxima, divides,
+// writes the scale and leaves every word zero.  A workgroup's arrival is issued after its maximum has returned,
+// so whoever sees a counter complete reads the maxima of all that were counted.
+constexpr int kScaleThreads = 1024;  // at most; launches that one trip of 512 threads per CU covers take 512
+constexpr unsigned kScaleGroups = 8;
+constexpr int kScaleLine = 32;  // words between the pairs: 128 bytes
+constexpr unsigned kScaleSingle = 32;  // launches of up to this many workgroups meet on one pair
+
 template <bool SWIGLU>
-__global__ __launch_bounds__(256) void tensor_scale_kernel(const uint16_t *x, const uint16_t *up, size_t ld, int rows,
-                                                           int K, float divisor, uint32_t *ws, float *out) {
-  __shared__ uint32_t wave_max[4];
+__global__ __launch_bounds__(kScaleThreads) void tensor_scale_kernel(const uint16_t *x, const uint16_t *up, size_t ld, int rows,
+                                                                      int K, float divisor, uint32_t *ws, float *out) {
+  __shared__ uint32_t wave_max[kScaleThreads / 64];
   const int cpr = K >> 3;  // 16-byte chunks per row
   const size_t total = (size_t)rows * cpr;
+  const bool dense = ld == (size_t)K;  // chunk c sits at x + 8 * c: no division per chunk
+  constexpr int U = SWIGLU ? 4 : 8;
   uint32_t m = 0u;
-  // four chunks per thread and trip, all loads first: the blocks end in two atomics on the same two
-  // words, which serialise, so a small tensor wants few blocks and still many loads in flight
   const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t c0 = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c0 < total; c0 += 4 * stride) {
-    uint4 g[4], u[4];
+  for (size_t c0 = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c0 < total; c0 += U * stride) {
+    uint4 g[U], u[U];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < U; ++j) {
       const size_t c = c0 + j * stride;
       g[j] = make_uint4(0, 0, 0, 0);
       u[j] = g[j];
       if (c < total) {
-        const size_t r = c / cpr, k = (c % cpr) << 3;
-        g[j] = *reinterpret_cast<const uint4 *>(x + r * ld + k);
-        if (SWIGLU) u[j] = *reinterpret_cast<const uint4 *>(up + r * ld + k);
+        size_t off = c << 3;
+        if (!dense) {
+          const size_t r = c / cpr;
+          off = r * ld + ((c - r * cpr) << 3);
+        }
+        g[j] = *reinterpret_cast<const uint4 *>(x + off);
+        if (SWIGLU) u[j] = *reinterpret_cast<const uint4 *>(up + off);
       }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {  // an absent chunk is zeros: act_fn(0) * 0 = 0 leaves the maximum alone
+    for (int j = 0; j < U; ++j) {  // an absent chunk is zeros: act_fn(0) * 0 = 0 leaves the maximum alone
       uint32_t t[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
       if (SWIGLU) {
         t[0] = swiglu_pair(g[j].x, u[j].x), t[1] = swiglu_pair(g[j].y, u[j].y);
@@ -1070,18 +1138,32 @@ __global__ __launch_bounds__(256) void tensor_scale_kernel(const uint16_t *x, co
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
   __syncthreads();
   if (threadIdx.x != 0) return;
-  for (int w = 1; w < 4; ++w) m = wave_max[w] > m ? wave_max[w] : m;
-  // atomics on one word serialise: a block whose maximum is no larger than what the word already
-  // holds (it only grows, so a value read earlier is a lower bound) has nothing to add
-  uint32_t old = __hip_atomic_load(ws, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (m > old) old = atomicMax(ws, m);
-  const uint32_t arrived = atomicAdd(ws + 1, 1u + (old >> 31));  // old < 2^31: the add waits for the line above
-  if (arrived != gridDim.x - 1) return;
-  const float amax = u2f(atomicMax(ws, 0u));
-  const float scale = amax / divisor;
+  for (int w = 1; w < (int)(blockDim.x >> 6); ++w) m = wave_max[w] > m ? wave_max[w] : m;
+  // Every step below waits for the one before it to return (about half a microsecond each), so there are as few
+  // as the protocol allows: maximum, arrival; the last arrival of a group arrives at the top; the last arrival
+  // there reads the groups' maxima.  Up to kScaleSingle workgroups meet on the top pair alone.
+  uint32_t *top = ws;
+  if (gridDim.x > kScaleSingle) {
+    const int grp = (int)blockIdx.x % kScaleGroups;
+    const uint32_t members = ((uint32_t)gridDim.x - (uint32_t)grp + kScaleGroups - 1u) / kScaleGroups;
+    uint32_t *gw = ws + (1 + grp) * kScaleLine;  // this group's (maximum, counter)
+    const uint32_t old = atomicMax(gw, m);
+    if (atomicAdd(gw + 1, 1u + (old >> 31)) != members - 1u) return;  // old < 2^31: the add waits for the maximum
+    if (atomicAdd(top + 1, 1u) != kScaleGroups - 1u) return;
+    // every group's last arrival has been counted, each after all of its group's maxima: read them, zero them
+    for (int q = 0; q < kScaleGroups; ++q) {
+      const uint32_t v = atomicExch(ws + (1 + q) * kScaleLine, 0u);
+      m = q == 0 ? v : (v > m ? v : m);
+      __hip_atomic_store(ws + (1 + q) * kScaleLine + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  } else {
+    const uint32_t old = atomicMax(top, m);
+    if (atomicAdd(top + 1, 1u + (old >> 31)) != gridDim.x - 1u) return;
+    m = atomicExch(top, 0u);
+  }
+  __hip_atomic_store(top + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const float scale = u2f(m) / divisor;
   *out = scale == 0.0f ? 1.0f : scale;
-  atomicExch(ws, 0u);
-  atomicExch(ws + 1, 0u);
 }
 
 // Per-segment maxima for grouped launches (rows sorted by segment): max |x|, or max |act_fn(gate) * up|,
@@ -1543,14 +1625,19 @@ int arcq_tensor_scale(const void *x, const void *up, int ld, int M, int K, float
   uint32_t *ws = static_cast<uint32_t *>(arcq::stream_workspace(arcq::kWsTensorScale, st, &status));
   if (!ws) return status;
   const size_t chunks = (size_t)M * (K >> 3);
-  int grid = (int)((chunks + 1023) / 1024 < 1024 ? (chunks + 1023) / 1024 : 1024);  // four chunks per thread
+  // at most one workgroup per CU; 512 threads x 8 chunks each while one trip of that covers the tensor (small
+  // tensors: fewer waves to meet at the end), 1024 threads beyond
+  const int threads = chunks <= (size_t)256 * 512 * 8 ? 512 : arcq::kScaleThreads;
+  const size_t per_wg = (size_t)threads * 8;
+  int grid = (int)std::min<size_t>(256, (chunks + per_wg - 1) / per_wg);
   if (grid < 1) grid = 1;  // M == 0: one block writes the scale of an empty tensor, 1
   if (up)
-    hipLaunchKernelGGL(arcq::tensor_scale_kernel<true>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(x),
-                       static_cast<const uint16_t *>(up), (size_t)ld, M, K, divisor, ws, d_scale);
+    hipLaunchKernelGGL(arcq::tensor_scale_kernel<true>, dim3(grid), dim3(threads), 0, st,
+                       static_cast<const uint16_t *>(x), static_cast<const uint16_t *>(up), (size_t)ld, M, K, divisor, ws, d_scale);
   else
-    hipLaunchKernelGGL(arcq::tensor_scale_kernel<false>, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(x),
-                       static_cast<const uint16_t *>(nullptr), (size_t)ld, M, K, divisor, ws, d_scale);
+    hipLaunchKernelGGL(arcq::tensor_scale_kernel<false>, dim3(grid), dim3(threads), 0, st,
+                       static_cast<const uint16_t *>(x), static_cast<const uint16_t *>(nullptr), (size_t)ld, M, K, divisor, ws,
+                       d_scale);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
 }

@@ -176,6 +176,66 @@ long long arcq_host_check_two_sided(int fmt, long n, long long *accepted, long l
   return bad;
 }
 
+// The quantizer's encode for a tensor scale g that is not a power of two, without forming y = x/g per element:
+// the block scale comes from RN(max|x| / g) (RN(x/g) is monotone in |x|, so that is max|y|), the codes from
+// x * R * (1 +- 2^-20) with R = RN(rg * r), rg = RN(1/g), r within an ulp of 1/s, through the RNE convert; where
+// the two codes differ, y = RN(x/g) is formed for that element and e2m1_resolve decides.  Checked against the
+// reference's e2m1_code(RN(RN(x/g) / s)) for every finite bf16 x with |x/g| <= 8s (and a sample beyond), every
+// block scale s, r off by -1, 0, +1 ulp, and tensor scales g = m / 2688 for every bf16 significand m (what
+// max|x| / 2688 can be) at several exponents plus n_random pseudo-random fp32 g.  Returns the number of wrong
+// codes; *accepted / *checked report how often the two conversions agreed.
+long long arcq_host_check_scaled_direct(int fmt, int n_random, long long *accepted, long long *checked) {
+  const int nscale = fmt == 0 ? 143 : 60;
+  const int n_struct = 128 * 3;
+  long long bad = 0, acc = 0, cnt = 0;
+#pragma omp parallel for schedule(dynamic, 4) reduction(+ : bad, acc, cnt)
+  for (int gi = 0; gi < n_struct + n_random; ++gi) {
+    float g;
+    if (gi < n_struct) {
+      const float mx = arcq::u2f(((uint32_t)(127 - 3 + 4 * (gi / 128)) << 23) | ((uint32_t)(gi % 128) << 16));
+      g = mx / 2688.0f;
+    } else {
+      uint64_t st = 0x9e3779b97f4a7c15ull * (uint64_t)(gi + 1);
+      st = st * 6364136223846793005ull + 1442695040888963407ull;
+      g = arcq::u2f(((uint32_t)(115 + (st >> 59) % 12) << 23) | ((uint32_t)(st >> 20) & 0x7fffffu));
+    }
+    const float rg = 1.0f / g;
+    for (int si = 0; si < nscale; ++si) {
+      const uint32_t sb = fmt == 0 ? (uint32_t)si : (uint32_t)(127 - 40 + si);
+      const float s = fmt == 0 ? arcq::nvfp4_scale_value(sb) : arcq::mxfp4_scale_value(sb);
+      const float r_exact = fmt == 0 ? 1.0f / s : arcq::u2f((254u << 23) - arcq::f2u(s));
+      for (uint32_t hb = 0; hb < 0x10000u; ++hb) {
+        if ((hb & 0x7f80u) == 0x7f80u) continue;  // inf / nan
+        const float x = arcq::bf16_bits_to_f32(hb);
+        const float y = x / g;                     // the reference's x32 (quantize.py:330)
+        const float ay = y < 0 ? -y : y;
+        if (!(ay <= 8.0f * s) && (hb & 0x7fu) != 0x2bu) continue;        // a sample of the saturating range
+        if (ay < 0x1p-8f * s && (hb & 0x7fu) != 0x2bu) continue;          // far below the first decision point
+        if (!(ay < 0x1p+100f) || (ay != 0.0f && ay < 0x1p-100f)) continue;  // such units are redone with IEEE divisions
+        const uint32_t exact = arcq::e2m1_code(y / s);
+        for (int d = (fmt == 0 ? -1 : 0); d <= (fmt == 0 ? 1 : 0); ++d) {
+          const float r = arcq::u2f(arcq::f2u(r_exact) + (uint32_t)d);
+          const float R = rg * r;
+          const float Ra = R * 0x1.00001p+0f, Rb = R * 0x1.ffffep-1f;
+          const uint32_t ca = arcq::e2m1_rne_hw_model(x * Ra), cb = arcq::e2m1_rne_hw_model(x * Rb);
+          ++cnt;
+          uint32_t got;
+          if (ca != cb) {
+            got = arcq::e2m1_resolve(arcq::div_bf16_by(x, g, rg), s, ca, cb);
+          } else {
+            ++acc;
+            got = (ca & 7u) == 0u ? 0u : ca;  // drop_negative_zeros
+          }
+          if (got != exact) ++bad;
+        }
+      }
+    }
+  }
+  *accepted = acc;
+  *checked = cnt;
+  return bad;
+}
+
 // 1/sqrt(a) as the RMSNorm kernel forms it (sqrt_from_estimate, rcp_from_estimate) against
 // 1.0f / sqrtf(a), with the hardware estimates modelled as the correctly rounded value moved by
 // -1, 0, +1 ulp.  a runs over n values spread across [2^-90, 2^100] plus a dense stretch.

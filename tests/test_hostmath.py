@@ -135,3 +135,19 @@ def test_rstd_from_hardware_estimates_is_exact(hm):
     hm.arcq_host_check_rstd.restype = ctypes.c_long
     hm.arcq_host_check_rstd.argtypes = [ctypes.c_long]
     assert hm.arcq_host_check_rstd(40_000_000) == 0
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_scaled_encode_without_per_element_division_is_exact(hm, fmt):
+    """the encode of units outside the residual range under an NVFP4 tensor scale: one division per unit (the
+    maximum), codes from x * RN(rg * r) * (1 +- 2^-20), e2m1_resolve on RN(x/g) where the two conversions differ --
+    against the reference's code of RN(RN(x/g) / s) for every bf16 x in reach of every block scale, tensor scales
+    max / 2688 for every bf16 significand of the maximum and pseudo-random ones, reciprocal off by -1/0/+1 ulp"""
+    hm.arcq_host_check_scaled_direct.restype = ctypes.c_longlong
+    hm.arcq_host_check_scaled_direct.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_longlong),
+                                                 ctypes.POINTER(ctypes.c_longlong)]
+    acc, cnt = ctypes.c_longlong(), ctypes.c_longlong()
+    bad = hm.arcq_host_check_scaled_direct(fmt, 1500, ctypes.byref(acc), ctypes.byref(cnt))
+    assert bad == 0, f"{bad} of {cnt.value}"
+    assert cnt.value > 250_000_000
+    assert acc.value / cnt.value > 0.99
