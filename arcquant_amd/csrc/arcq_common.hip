@@ -92,6 +92,7 @@ const Tuning &tuning() {
     Tuning v;
     if (const char *e = getenv("ARCQ_GEMM_KERNEL")) v.gemm_kernel = atoi(e);
     if (const char *e = getenv("ARCQ_GEMM_SPLITK")) v.gemm_splitk = atoi(e);
+    if (const char *e = getenv("ARCQ_GEMM_PERSIST")) v.gemm_persist = atoi(e);
     if (const char *e = getenv("ARCQ_QUANT_GRID")) v.quant_grid = atoi(e);
     if (const char *e = getenv("ARCQ_QUANT_KERNEL")) v.quant_kernel = atoi(e);
     if (const char *e = getenv("ARCQ_KV_DECODE_SPLITS")) v.kv_decode_splits = atoi(e);

@@ -151,6 +151,30 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, const v16f &acc,
   }
 }
 
+// One 32x32 accumulator tile that lies inside C, with 16-byte stores: lanes r and r + 32 hold the two halves of
+// eight consecutive columns of row r for every q; one half-wave swap (v_permlane32_swap) per register pair gives
+// the lower lane all eight columns of an even q and the upper lane those of the odd q behind it.
+// c: this lane's address for q = 0 (row m0 + lane % 32, column n0 + 8 * (lane / 32)); res: the same into the residual, or NULL.
+__device__ __forceinline__ void store_tile_rows16(const v16f &acc, uint16_t *c, const uint16_t *res, float alpha) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {  // q = 2h (lower lanes) and 2h + 1 (upper lanes)
+    const uint32_t e0 = pack_bf16_rne(acc[8 * h] * alpha, acc[8 * h + 1] * alpha);
+    const uint32_t e1 = pack_bf16_rne(acc[8 * h + 2] * alpha, acc[8 * h + 3] * alpha);
+    const uint32_t o0 = pack_bf16_rne(acc[8 * h + 4] * alpha, acc[8 * h + 5] * alpha);
+    const uint32_t o1 = pack_bf16_rne(acc[8 * h + 6] * alpha, acc[8 * h + 7] * alpha);
+    // swap(upper lanes of the first operand, lower lanes of the second): lower lanes end up with (own even q,
+    // partner's even q), upper lanes with (partner's odd q, own odd q)
+    const auto s0 = __builtin_amdgcn_permlane32_swap(e0, o0, false, false);
+    const auto s1 = __builtin_amdgcn_permlane32_swap(e1, o1, false, false);
+    uint4 v = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+    if (res) {
+      const uint4 rv = *reinterpret_cast<const uint4 *>(res + 16 * h);
+      v = make_uint4(add_bf16_pair(v.x, rv.x), add_bf16_pair(v.y, rv.y), add_bf16_pair(v.z, rv.z), add_bf16_pair(v.w, rv.w));
+    }
+    *reinterpret_cast<uint4 *>(c + 16 * h) = v;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Baseline kernels: operands straight from global memory into registers.  Correct for every
 // shape the entry point accepts; the tuned kernels below are checked against the same oracle.
@@ -504,10 +528,15 @@ struct MfmaReadPattern {
   }
 };
 
-template <int WN, int WM, int NS = 2, int NWM = 2>
+template <int WN, int WM, int NS = 2, int NWM = 2, bool PERSIST = false>
 __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
   // waves: 2 along N x NWM along M (wave = n + 2 * m), each with WN x WM accumulator tiles of 32 x 32
   constexpr int BN = 64 * WN, BM = 32 * WM * NWM, NW = 2 * NWM;
+  // PERSIST (eight-wave tiles, plain launches): at most one workgroup per CU walks the tiles of its XCD's run.
+  // The stages and the scale pairs keep alternating across tiles, so the first stage of the next tile is
+  // requested during the last K step of the current one, and the finished tile leaves straight from the
+  // accumulator registers (no LDS, no barrier) while those requests are on their way.
+  static_assert(!PERSIST || (NWM == 4 && NS == 2 && WN == 4 && WM == 2), "persistent workgroups are built on the 256x256 requesting-wave layout");
   // Eight waves (two per SIMD): the first wave of every SIMD requests the whole next stage, the second one
   // goes straight to its MFMAs, so the matrix pipe works while the requests queue up in the load unit.
   constexpr bool kLoaderWaves = NWM == 4 && NS == 2;
@@ -525,16 +554,26 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
   // tile of this workgroup: consecutive workgroup ids go to different XCDs (8 of them, each with
   // its own L2), so hand each XCD a contiguous run of tiles that walk down M for a fixed weight tile
   int lin;
+  int run_left = 0, run_step = 0;  // PERSIST: tiles of this XCD's run still ahead of `lin`, distance between this workgroup's tiles
   if (p.seg) {
     if (!enter_segment<BM, BN, 32>(p, lin)) return;
   } else {
     const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
     const int per_xcd = (total + 7) >> 3;
-    lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (lin >= total) return;
+    if constexpr (PERSIST) {
+      const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+      run_step = gridDim.x >> 3;
+      const int run_end = min(total, (xcd + 1) * per_xcd);
+      lin = xcd * per_xcd + slot;
+      if (lin >= run_end) return;
+      run_left = run_end - lin;
+    } else {
+      lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+      if (lin >= total) return;
+    }
   }
   const int tiles_m = (p.M + BM - 1) / BM;
-  const int n_base = (lin / tiles_m) * BN, m_base = (lin % tiles_m) * BM;
+  int n_base = (lin / tiles_m) * BN, m_base = (lin % tiles_m) * BM;
 
   const int nk = (p.Kp + 255) >> 8;
   const bool short_last = (p.Kp & 255) != 0;  // then the last step has 4 valid blocks (K' % 256 == 128)
@@ -545,14 +584,24 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
   // With requesting waves the addresses are a wave-uniform base (operand + K offset) plus a 32-bit byte
   // offset per lane (the host sends operands of 4 GiB and more to the four-wave kernels).
   constexpr int NPW = kLoaderWaves ? 1 : BN / RPI, NPX = kLoaderWaves ? 1 : BM / RPI;
-  constexpr int NOW = kLoaderWaves ? BN / RPI : 1, NOX = kLoaderWaves ? BM / RPI : 1;
+  // (persistent workgroups see whole tiles only: no row is clamped, the rows of one lane are RPI * kbytes apart,
+  // and one offset per operand is enough: the multiples go into the scalar base)
+  constexpr int NOW = kLoaderWaves && !PERSIST ? BN / RPI : 1, NOX = kLoaderWaves && !PERSIST ? BM / RPI : 1;
   const uint8_t *wsrc[NPW], *xsrc[NPX];
   uint32_t wvo[NOW], xvo[NOX];
+  uint32_t wsvo = 0, xsvo = 0;
+  const int npairs = (nk + 1) >> 1;
+  const int sc_shift = max(0, npairs * 16 - ksc);
+  auto lane_offsets = [&](int nb, int mb) {  // requesting waves: this lane's byte offsets into the operands for a tile
+#pragma unroll
+    for (int i = 0; i < NOW; ++i) wvo[i] = (uint32_t)min(nb + RPI * i + ld_row, p.N - 1) * (uint32_t)kbytes + ld_q * 16;
+#pragma unroll
+    for (int i = 0; i < NOX; ++i) xvo[i] = (uint32_t)min(mb + RPI * i + ld_row, p.M - 1) * (uint32_t)kbytes + ld_q * 16;
+    wsvo = (uint32_t)min(nb + 64 * min(wave, BN / 64 - 1) + lane, p.N - 1) * (uint32_t)ksc;
+    xsvo = (uint32_t)min(mb + 64 * min(wave, BM / 64 - 1) + lane, p.M - 1) * (uint32_t)ksc;
+  };
   if constexpr (kLoaderWaves) {
-#pragma unroll
-    for (int i = 0; i < BN / RPI; ++i) wvo[i] = (uint32_t)min(n_base + RPI * i + ld_row, p.N - 1) * (uint32_t)kbytes + ld_q * 16;
-#pragma unroll
-    for (int i = 0; i < BM / RPI; ++i) xvo[i] = (uint32_t)min(m_base + RPI * i + ld_row, p.M - 1) * (uint32_t)kbytes + ld_q * 16;
+    lane_offsets(n_base, m_base);
   } else {
 #pragma unroll
     for (int i = 0; i < BN / RPI; ++i)
@@ -566,15 +615,9 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
   // activations to wave (j+BN/64)%NW; with requesting waves, instruction j of either operand to wave j.
   // If the row ends inside the last pair, the 16-byte window is
   // shifted back to end at the row end (sc_shift bytes; K' % 128 == 0 makes it a multiple of 4).
-  const int npairs = (nk + 1) >> 1;
-  const int sc_shift = max(0, npairs * 16 - ksc);
   constexpr int NPS = kLoaderWaves ? 1 : BN / 64, NPT = kLoaderWaves ? 1 : BM / 64;
   const uint8_t *wssrc[NPS], *xssrc[NPT];
-  uint32_t wsvo = 0, xsvo = 0;
-  if constexpr (kLoaderWaves) {
-    wsvo = (uint32_t)min(n_base + 64 * min(wave, BN / 64 - 1) + lane, p.N - 1) * (uint32_t)ksc;
-    xsvo = (uint32_t)min(m_base + 64 * min(wave, BM / 64 - 1) + lane, p.M - 1) * (uint32_t)ksc;
-  } else {
+  if constexpr (!kLoaderWaves) {
 #pragma unroll
     for (int j = 0; j < BN / 64; ++j) wssrc[j] = p.b_scales + (size_t)min(n_base + 64 * j + lane, p.N - 1) * ksc;
 #pragma unroll
@@ -585,20 +628,26 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
   const uint32_t lws0 = (uint32_t)reinterpret_cast<uintptr_t>(sWs);
   const uint32_t lxs0 = (uint32_t)reinterpret_cast<uintptr_t>(sXs);
 
-  auto issue = [&](int kt) {
-    const int st = kt & (NS - 1);
+  // sb / pb: K steps and scale pairs of the tiles this workgroup has finished (0 unless PERSIST): the stage of a
+  // step and of a pair alternate across tiles
+  int step_base = 0, pair_base = 0;
+  auto issue = [&](int kt, int sb, int pb) {
+    const int st = (kt + sb) & (NS - 1);
     // a short last step has only chunks 0..3: fetch those twice; the products of the absent blocks
     // are zeroed in compute()
     const bool clip = short_last && kt == nk - 1;
     if constexpr (kLoaderWaves) {
       const uint8_t *wb = p.b_codes + kt * 128, *xb = p.a_codes + kt * 128;
       const uint32_t back = (clip && ld_q >= 4) ? 64u : 0u;
+      const size_t rows_step = PERSIST ? (size_t)RPI * kbytes : 0;
 #pragma unroll
-      for (int i = 0; i < BN / RPI; ++i) lds_dma16_at(wb, wvo[i] - back, lw0 + st * (BN * 128) + i * (RPI * 128));
+      for (int i = 0; i < BN / RPI; ++i)
+        lds_dma16_at(wb + i * rows_step, wvo[PERSIST ? 0 : i] - back, lw0 + st * (BN * 128) + i * (RPI * 128));
 #pragma unroll
-      for (int i = 0; i < BM / RPI; ++i) lds_dma16_at(xb, xvo[i] - back, lx0 + st * (BM * 128) + i * (RPI * 128));
+      for (int i = 0; i < BM / RPI; ++i)
+        lds_dma16_at(xb + i * rows_step, xvo[PERSIST ? 0 : i] - back, lx0 + st * (BM * 128) + i * (RPI * 128));
       if ((kt & 1) == 0) {  // scales of steps kt and kt+1
-        const int pair = kt >> 1, sst = pair & (NS - 1);
+        const int pair = kt >> 1, sst = (pair + pb) & (NS - 1);
         const int soff = pair * 16 - (pair == npairs - 1 ? sc_shift : 0);
         if (wave < BN / 64) lds_dma16_at(p.b_scales + soff, wsvo, lws0 + sst * (BN * 16) + wave * 1024);
         if (wave < BM / 64) lds_dma16_at(p.a_scales + soff, xsvo, lxs0 + sst * (BM * 16) + wave * 1024);
@@ -610,7 +659,7 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
 #pragma unroll
     for (int i = 0; i < NPX; ++i) lds_dma16(xsrc[i] + koff, lx0 + st * (BM * 128) + i * (RPI * 128));
     if ((kt & 1) == 0) {  // scales of steps kt and kt+1
-      const int pair = kt >> 1, sst = pair & (NS - 1);
+      const int pair = kt >> 1, sst = (pair + pb) & (NS - 1);
       const int soff = pair * 16 - (pair == npairs - 1 ? sc_shift : 0);
 #pragma unroll
       for (int j = 0; j < NPS; ++j)
@@ -647,7 +696,7 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
   // one read behind each of the first MFMAs), so neither their issue nor their latency idles the matrix pipe.
   auto compute = [&](int kt, auto tail) {
     constexpr bool TAIL = decltype(tail)::value;
-    const int st = kt & (NS - 1), sst = (kt >> 1) & (NS - 1);
+    const int st = (kt + step_base) & (NS - 1), sst = ((kt >> 1) + pair_base) & (NS - 1);
     const uint4 *cw = sW + st * (BN * 8), *cx = sX + st * (BM * 8);
     // this lane's four scale bytes of the step inside the row's 16-byte pair window; a lane whose
     // blocks are absent (short last step) may point past it and is clamped: its operands are zero
@@ -715,7 +764,9 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
         asm volatile("s_waitcnt vmcnt(13)" ::: "memory");
       else
         asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-    } else {
+    } else if (!PERSIST || wave < NLW) {
+      // (persistent workgroups: the waves that request nothing have only a finished tile's stores outstanding,
+      // and those may drain behind the next tile's first steps)
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
@@ -725,19 +776,103 @@ __global__ __launch_bounds__(128 * NWM) void gemm_mxfp4_tiled(GemmParams p) {
   const bool requests = wave < NLW;
 #pragma unroll
   for (int a = 0; a < NS - 1; ++a)
-    if (kt_beg + a < kt_end && requests) issue(kt_beg + a);
-  for (int kt = kt_beg; kt < nfull; ++kt) {
-    wait_step(kt_end - 1 - kt);  // the stage of step kt is complete; everyone is done with the stage of step kt-1
-    if (kt + NS - 1 < kt_end && requests) issue(kt + NS - 1);
-    compute(kt, std::false_type{});
+    if (kt_beg + a < kt_end && requests) issue(kt_beg + a, 0, 0);
+  if constexpr (!PERSIST) {
+    for (int kt = kt_beg; kt < nfull; ++kt) {
+      wait_step(kt_end - 1 - kt);  // the stage of step kt is complete; everyone is done with the stage of step kt-1
+      if (kt + NS - 1 < kt_end && requests) issue(kt + NS - 1, 0, 0);
+      compute(kt, std::false_type{});
+    }
+    if (tail && kt_beg < kt_end) {
+      wait_step(0);
+      compute(nk - 1, std::true_type{});
+    }
+    store_workgroup_tile<WN, WM, NWM>(p, acc, reinterpret_cast<uint8_t *>(sW), reinterpret_cast<uint8_t *>(sX), m_base,
+                                      n_base, wave, lane);
+  } else {
+    // (the host sends only problems made of whole tiles here: M % BM == 0, N % BN == 0)
+    const float alpha = effective_alpha(p);
+    for (;;) {
+      const bool more = run_left > run_step;  // this workgroup has another tile
+      const int cur_n = n_base, cur_m = m_base;
+      auto request_next_tile = [&]() {  // during the last step: the next tile's first stage goes out before it is multiplied
+        if (!more) return;
+        lin += run_step;
+        n_base = (lin / tiles_m) * BN;
+        m_base = (lin % tiles_m) * BM;
+        if (requests) {
+          lane_offsets(n_base, m_base);
+          issue(0, step_base + nk, pair_base + npairs);
+        }
+      };
+      for (int kt = 0; kt < nfull; ++kt) {
+        wait_step(0);
+        if (kt + 1 < nk) {
+          if (requests) issue(kt + 1, step_base, pair_base);
+        } else {
+          request_next_tile();
+        }
+        compute(kt, std::false_type{});
+      }
+      if (tail) {
+        wait_step(0);
+        request_next_tile();
+        compute(nk - 1, std::true_type{});
+      }
+      // The finished tile leaves through the stage that the last step has just been multiplied from: it stays
+      // free until the next tile's second step is requested, which happens behind the barrier of its first
+      // step, i.e. after every wave's epilogue.  Each wave transposes its own 32-row slabs in an 8 KB piece of
+      // that stage (wave-local: the one barrier here only says that everyone is done reading operands), so that
+      // every store instruction writes whole rows of the wave tile, 16 bytes per lane.
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+      {
+        const int st_last = (nk - 1 + step_base) & 1;
+        uint8_t *region = reinterpret_cast<uint8_t *>(wave < 4 ? sW + st_last * (BN * 8) : sX + st_last * (BM * 8)) + (wave & 3) * 8192;
+        static_assert(BN * 128 >= 4 * 8192 && BM * 128 >= 4 * 8192 && 32 * 64 * WN == 8192, "8 KB per wave inside one stage of either operand");
+        constexpr int RB = 64 * WN, LPR = 4 * WN;   // bytes per row of the wave tile, lanes per row at 16 bytes each
+        // (the lane number is made opaque here: the LDS addresses below do not depend on the tile, and hoisted out
+        // of the tile loop they would be spilled and reloaded one by one)
+        int lane_e = lane;
+        asm volatile("" : "+v"(lane_e));
+        const int r_e = lane_e & 31, kh_e = lane_e >> 5;
+        const int rr = lane_e / LPR, t = lane_e % LPR;
+#pragma unroll
+        for (int j = 0; j < WM; ++j) {
+          const int sw = (r_e & (LPR - 1)) << 1;
+#pragma unroll
+          for (int i = 0; i < WN; ++i) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const v16f &a = acc[i][j];
+              const int c = 8 * i + 2 * q + kh_e;  // 8-byte chunk of the row
+              *reinterpret_cast<uint2 *>(region + r_e * RB + ((c ^ sw) << 3)) =
+                  make_uint2(pack_bf16_rne(a[4 * q] * alpha, a[4 * q + 1] * alpha), pack_bf16_rne(a[4 * q + 2] * alpha, a[4 * q + 3] * alpha));
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+          }
+          uint16_t *cbase = p.c + (size_t)(cur_m + wm0 + 32 * j) * p.N + cur_n + wn0 + 8 * t;
+#pragma unroll
+          for (int it = 0; it < (32 * LPR) / 64; ++it) {
+            const int m = it * (64 / LPR) + rr;
+            const int swr = (m & (LPR - 1)) << 1;
+            uint4 v = *reinterpret_cast<const uint4 *>(region + m * RB + (((2 * t) ^ swr) << 3));
+            if (p.residual) {
+              const uint4 rv = *reinterpret_cast<const uint4 *>(p.residual + (cbase - p.c) + (size_t)m * p.N);
+              v = make_uint4(add_bf16_pair(v.x, rv.x), add_bf16_pair(v.y, rv.y), add_bf16_pair(v.z, rv.z), add_bf16_pair(v.w, rv.w));
+            }
+            *reinterpret_cast<uint4 *>(cbase + (size_t)m * p.N) = v;
+          }
+        }
+      }
+      if (!more) break;
+      run_left -= run_step;
+      step_base += nk;
+      pair_base += npairs;
+    }
   }
-  if (tail && kt_beg < kt_end) {
-    wait_step(0);
-    compute(nk - 1, std::true_type{});
-  }
-
-  store_workgroup_tile<WN, WM, NWM>(p, acc, reinterpret_cast<uint8_t *>(sW), reinterpret_cast<uint8_t *>(sX), m_base,
-                                    n_base, wave, lane);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1193,6 +1328,18 @@ int launch_mxfp4_tiled(const GemmParams &p, hipStream_t st) {
   return ARCQ_OK;
 }
 
+// The eight-wave tiles as persistent workgroups, one per CU at most (plain launches: no expert segments, no fused
+// SwiGLU, K not cut)
+template <int WN, int WM>
+int launch_mxfp4_persistent(const GemmParams &p, hipStream_t st) {
+  constexpr int BN = 64 * WN, BM = 32 * WM * 4;
+  const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  const int grid = std::min(256, ((total + 7) / 8) * 8);  // whole groups of 8: one slot per XCD and group
+  hipLaunchKernelGGL((gemm_mxfp4_tiled<WN, WM, 2, 4, true>), dim3(grid), dim3(512), 0, st, p);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
 // Split-K for few rows of activations and narrow layers: a 128x64 tile grid alone leaves most CUs idle
 // (N = 4096, M = 64: 32 workgroups), so K is cut into slices, one workgroup per (tile, slice), each
 // writing its fp32 partial tile; this kernel adds the slices in order and writes bf16.  The kernel
@@ -1345,10 +1492,16 @@ int run_gemm(GemmParams p, const GemmPlan &plan, int fmt, float *scratch, hipStr
   if (fmt == ARCQ_FMT_MXFP4) {
     // the eight-wave kernels address an operand's rows with 32-bit byte offsets from its base
     const bool wide = (size_t)std::max(p.M, p.N) * (size_t)(p.Kp >> 1) >= ((size_t)1 << 32);
+    // persistent workgroups: plain launches over whole tiles
+    // and more of them than one round of workgroups: with a single tile per CU there is nothing to overlap
+    // (gate_up at M = 4096, seven tiles per CU: 333 -> 325 us; qkv, one and a half: 77.5 -> 74.9; one round: 1-3 % slower)
+    const bool persist = !p.seg && !p.swiglu && tuning().gemm_persist != 0 && p.M % 256 == 0 && p.N % 256 == 0 &&
+                         (long)(p.M / 256) * (p.N / 256) > 256;
     switch (wide && plan.kernel == 84 ? 44 : (wide && plan.kernel == 82 ? 42 : plan.kernel)) {
       case 44: return launch_mxfp4_tiled<4, 4>(p, st);
-      case 84: return launch_mxfp4_tiled<4, 2, 2, 4>(p, st);  // 256x256 tile, eight waves of 128x64
-      case 82: return launch_mxfp4_tiled<4, 1, 2, 4>(p, st);  // 256x128 tile, eight waves of 128x32
+      // 256x256 tile, eight waves of 128x64, and 256x128 tile, eight waves of 128x32
+      case 84: return persist ? launch_mxfp4_persistent<4, 2>(p, st) : launch_mxfp4_tiled<4, 2, 2, 4>(p, st);
+      case 82: return launch_mxfp4_tiled<4, 1, 2, 4>(p, st);
       case 42: return launch_mxfp4_tiled<4, 2>(p, st);
       case 224: return launch_mxfp4_tiled<2, 2, 4>(p, st);
       case 22: return launch_mxfp4_tiled<2, 2>(p, st);

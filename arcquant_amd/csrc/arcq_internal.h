@@ -51,6 +51,7 @@ int noalloc_prepare();
 //   ARCQ_GEMM_KERNEL=<WN><WM>   force a GEMM tile (84 / 82 = 256x256 / 256x128 as eight waves, 44, 42, 22, 21, 11; 214 / 224 = four-stage
 //                               ring; 1 = skinny, 0 = direct); a number the format has no kernel for is ignored
 //   ARCQ_GEMM_SPLITK=<slices>   force split-K for M <= 512 (1 = never split)
+//   ARCQ_GEMM_PERSIST=<0|1>     0 = the eight-wave MXFP4 tiles as one workgroup per tile instead of persistent workgroups
 //   ARCQ_QUANT_GRID=<n>         workgroups of the row quantizers
 //   ARCQ_QUANT_KERNEL=<1|2|3>   1 = never, 2 = always take the wave-per-row quantizer where it has an instance;
 //                               3 = the four-units-per-thread kernel of the rows beyond 16384 channels from 1024 channels on
@@ -59,6 +60,7 @@ int noalloc_prepare();
 struct Tuning {
   int gemm_kernel = -1;
   int gemm_splitk = 0;
+  int gemm_persist = 1;
   int quant_grid = 0;
   int quant_kernel = 0;
   int kv_decode_splits = 0;
