@@ -2,6 +2,7 @@
 
     python -m arcquant_amd.build            # build if stale
     python -m arcquant_amd.build --force    # rebuild even if up to date
+    python -m arcquant_amd.build --experiments   # with the measured-and-not-taken kernel variants (ARCQ_GEMM_KERNEL)
 
 hipcc cross-compiles for gfx950 without a GPU present.  The built libraries live next to the
 sources (arcquant_amd/csrc/) so that they travel with the tree.
@@ -45,12 +46,14 @@ def _stale(target: str, deps) -> bool:
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build_hip(force: bool = False, verbose: bool = False) -> str:
+def build_hip(force: bool = False, verbose: bool = False, experiments: bool = False) -> str:
     srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
     deps = srcs + [os.path.join(CSRC, h) for h in ("arcq_math.h", "arcq_internal.h", "arcq_swiglu.h")] + [
         os.path.join(HERE, "..", "include", "arcq.h")]
     if force or _stale(HIP_LIB, deps):
-        cmd = [_hipcc(), *HIPCC_FLAGS, "-o", HIP_LIB, *srcs]
+        # --experiments: also the kernel variants that were measured and not taken (reached only through
+        # ARCQ_GEMM_KERNEL; the counter summaries under profiles/ that name one were made with such a build)
+        cmd = [_hipcc(), *HIPCC_FLAGS, *(["-DARCQ_EXPERIMENTS"] if experiments else []), "-o", HIP_LIB, *srcs]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
@@ -67,9 +70,9 @@ def build_probe(force: bool = False, verbose: bool = False) -> str:
     return PROBE_LIB
 
 
-def build_all(force: bool = False, verbose: bool = False):
-    return (build_hip(force, verbose), build_probe(force, verbose))
+def build_all(force: bool = False, verbose: bool = False, experiments: bool = False):
+    return (build_hip(force or experiments, verbose, experiments), build_probe(force, verbose))
 
 
 if __name__ == "__main__":
-    print(build_all(force="--force" in sys.argv, verbose=True))
+    print(build_all(force="--force" in sys.argv, verbose=True, experiments="--experiments" in sys.argv))

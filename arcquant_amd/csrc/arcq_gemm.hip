@@ -1106,6 +1106,186 @@ __global__ __launch_bounds__(128 * NWM) void gemm_nvfp4_tiled(GemmParams p) {
                                     n_base, wave, lane);
 }
 
+#ifdef ARCQ_EXPERIMENTS
+// ---------------------------------------------------------------------------------------------
+// EXPERIMENT (built only with -DARCQ_EXPERIMENTS, reached only through ARCQ_GEMM_KERNEL=86 / 46; measured slower than
+// the kernel above: 963 against 826 us on gate_up at M = 4096).
+// NVFP4 at large M: every operand value is decoded ONCE per workgroup.  In the kernel above each wave decodes
+// the operand rows it multiplies, so a weight row is decoded by every wave along M and an activation row by
+// every wave along N, and the decode instructions (six per MFMA) share the issue slots of the one wave per SIMD
+// with the MFMAs.  Here the workgroup's eight waves (2 along N x 4 along M, wave tile 128 x 64, two waves per
+// SIMD) first act as decoders: per K step of 64 elements a thread takes 32 codes of one weight row and 32 of
+// one activation row straight from global memory (16 bytes and two scale bytes each), decodes them exactly to
+// fp16 (code value x block scale has six significant bits) and writes them into an fp16 tile in LDS -- two
+// stages of 2 x 256 rows x 128 bytes -- and then as multipliers: v_mfma_f32_32x32x16_f16 on 16-byte operand
+// reads from that tile, two decode instructions per MFMA instead of six.  The decode of step t+1 is interleaved
+// with the MFMAs of step t, its codes were requested during step t-1; one barrier per step.
+// Requires K' % 128 == 0.
+// ---------------------------------------------------------------------------------------------
+template <int NWM>  // waves along M: 4 = eight waves of 128 x 64 (two per SIMD), 2 = four waves of 128 x 128
+__global__ __launch_bounds__(128 * NWM) void gemm_nvfp4_lds16(GemmParams p) {
+  constexpr int WN = 4, WM = 8 / NWM, BN = 256, BM = 256, NT = 128 * NWM, IPT = 512 / NT;  // IPT: decoder items per thread and operand
+  __shared__ uint4 sT[2 * (BN + BM) * 8];  // stage s: fp16 weights [BN rows x 8 chunks] at s*(BN+BM)*8, activations behind them
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kbytes = p.Kp >> 1, ksc = p.Kp >> 4;
+
+  int lin;
+  if (p.seg) {
+    if (!enter_segment<BM, BN, 16>(p, lin)) return;
+  } else {
+    const int total = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+    const int per_xcd = (total + 7) >> 3;
+    lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (lin >= total) return;
+  }
+  const int tiles_m = (p.M + BM - 1) / BM;
+  const int n_base = (lin / tiles_m) * BN, m_base = (lin % tiles_m) * BM;
+  const int nk = p.Kp >> 6;  // K steps of 64 elements: 32 code bytes and 4 scale bytes per row
+
+  // ---- decoder role: item (row, half h of the step's 64 elements) of either tile; a thread takes items tid + it * NT
+  const int d_h = tid & 1;
+  int d_row[IPT], d_swz[IPT];
+  const uint8_t *wc[IPT], *xc[IPT], *wsc[IPT], *xsc[IPT];
+  // chunk c (16 bytes = 8 fp16) of row `row` sits at row * 8 + (c ^ ((row >> 1) & 7)): rows two apart use different
+  // chunk slots and neighbouring rows different halves of the banks, so neither the decoders' 16-byte writes nor the
+  // multipliers' 16-byte reads (32 consecutive rows, one chunk) collide
+#pragma unroll
+  for (int it = 0; it < IPT; ++it) {
+    d_row[it] = (tid + it * NT) >> 1;
+    d_swz[it] = (d_row[it] >> 1) & 7;
+    wc[it] = p.b_codes + (size_t)min(n_base + d_row[it], p.N - 1) * kbytes + 16 * d_h;
+    xc[it] = p.a_codes + (size_t)min(m_base + d_row[it], p.M - 1) * kbytes + 16 * d_h;
+    wsc[it] = p.b_scales + (size_t)min(n_base + d_row[it], p.N - 1) * ksc + 2 * d_h;
+    xsc[it] = p.a_scales + (size_t)min(m_base + d_row[it], p.M - 1) * ksc + 2 * d_h;
+  }
+  struct Codes { uint4 w[IPT], x[IPT]; uint32_t ws[IPT], xs[IPT]; };
+  auto request = [&](int kt, Codes &c) {
+#pragma unroll
+    for (int it = 0; it < IPT; ++it) {
+      c.w[it] = *reinterpret_cast<const uint4 *>(wc[it] + 32 * kt);
+      c.x[it] = *reinterpret_cast<const uint4 *>(xc[it] + 32 * kt);
+      c.ws[it] = *reinterpret_cast<const uint16_t *>(wsc[it] + 4 * kt);
+      c.xs[it] = *reinterpret_cast<const uint16_t *>(xsc[it] + 4 * kt);
+    }
+  };
+  // dword D (8 codes) of a thread's 32 codes + its block's scale byte -> chunk 4 * d_h + D of the row's fp16 tile
+  // (dwords 0, 1 belong to the first of the two blocks, 2, 3 to the second)
+  auto decode_dword = [&](const uint4 &q, uint32_t two_scales, uint4 *tile_row, int d_swz, auto dsel) {
+    constexpr int D = decltype(dsel)::value;
+    const uint32_t sp = nv_scale_pair_f16((two_scales & 0xffu) | ((two_scales & 0xff00u) << 8));  // (block 0, block 1) as fp16
+    const uint32_t c = D == 0 ? q.x : D == 1 ? q.y : D == 2 ? q.z : q.w;
+    const v8h v = D < 2 ? decode8_nvfp4_f16<false>(c, sp) : decode8_nvfp4_f16<true>(c, sp);
+    tile_row[(4 * d_h + D) ^ d_swz] = __builtin_bit_cast(uint4, v);
+  };
+  auto decode_part = [&](const Codes &c, int stage, auto dsel) {  // a quarter of a step: 16 * IPT VALU instructions, 2 * IPT LDS writes
+    uint4 *base = sT + stage * ((BN + BM) * 8);
+#pragma unroll
+    for (int it = 0; it < IPT; ++it) {
+      decode_dword(c.w[it], c.ws[it], base + d_row[it] * 8, d_swz[it], dsel);
+      decode_dword(c.x[it], c.xs[it], base + BN * 8 + d_row[it] * 8, d_swz[it], dsel);
+    }
+  };
+  auto decode_step = [&](const Codes &c, int stage) {
+    decode_part(c, stage, std::integral_constant<int, 0>{});
+    decode_part(c, stage, std::integral_constant<int, 1>{});
+    decode_part(c, stage, std::integral_constant<int, 2>{});
+    decode_part(c, stage, std::integral_constant<int, 3>{});
+  };
+
+  // ---- multiplier role
+  const int r = lane & 31, kh = lane >> 5;
+  const int swz = (r >> 1) & 7;
+  const int wn0 = (wave & 1) * 32 * WN, wm0 = (wave >> 1) * 32 * WM;
+  int w_rd[4], x_rd[4];  // chunk 2 * ks + kh of this lane's row in operand tile 0, per sub-step of 16 elements
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    w_rd[ks] = (wn0 + r) * 8 + ((2 * ks + kh) ^ swz);
+    x_rd[ks] = BN * 8 + (wm0 + r) * 8 + ((2 * ks + kh) ^ swz);
+  }
+  v16f acc[WN][WM];
+#pragma unroll
+  for (int i = 0; i < WN; ++i)
+#pragma unroll
+    for (int j = 0; j < WM; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  auto lds_sync = [&]() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+  };
+
+  Codes ca, cb;  // the codes of the next step and of the one after it
+  request(0, ca);
+  if (nk > 1) request(1, cb);
+  decode_step(ca, 0);
+  lds_sync();
+  // One K step: the MFMAs of step kt and, if MORE, the decode of step kt + 1 (codes in cb, requested a step ago)
+  // into the other stage.  MORE is a compile-time flag so that a sub-step stays one basic block and the MFMAs,
+  // the decode instructions and the LDS traffic can be interleaved in it.
+  auto step = [&](int kt, auto more_t) {
+    constexpr bool MORE = decltype(more_t)::value;
+    const uint4 *t = sT + (kt & 1) * ((BN + BM) * 8);
+    uint4 wq[2][WN], xq[2][WM];
+    auto fetch = [&](int ks, int b) {
+#pragma unroll
+      for (int i = 0; i < (WN > WM ? WN : WM); ++i) {
+        if (i < WM) xq[b][i] = t[x_rd[ks] + i * 256];
+        if (i < WN) wq[b][i] = t[w_rd[ks] + i * 256];
+      }
+    };
+    fetch(0, 0);
+    // a quarter of the next step's decode (2 x (4 converts + 4 multiplies), two 16-byte LDS writes) rides behind the
+    // eight MFMAs of every sub-step: one MFMA, two decode instructions, and the operand reads of the next sub-step
+#define ARCQ_L16_SUBSTEP(KS)                                                                                     \
+  {                                                                                                              \
+    if (KS < 3) fetch(KS + 1, (KS + 1) & 1);                                                                     \
+    if (MORE) decode_part(cb, (kt + 1) & 1, std::integral_constant<int, KS>{});                                  \
+    _Pragma("unroll") for (int i = 0; i < WN; ++i) _Pragma("unroll") for (int j = 0; j < WM; ++j)                \
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, wq[KS & 1][i]),               \
+                                                          __builtin_bit_cast(v8h, xq[KS & 1][j]), acc[i][j], 0, 0, 0); \
+    _Pragma("unroll") for (int g = 0; g < WN * WM; ++g) {                                                        \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                         \
+      if (MORE) __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);                                               \
+      if (KS < 3 && g < WN + WM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                              \
+      if (MORE && g >= WN * WM - 2 * IPT) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                     \
+    }                                                                                                            \
+    __builtin_amdgcn_sched_barrier(0);                                                                           \
+  }
+    ARCQ_L16_SUBSTEP(0)
+    ARCQ_L16_SUBSTEP(1)
+    ARCQ_L16_SUBSTEP(2)
+    ARCQ_L16_SUBSTEP(3)
+#undef ARCQ_L16_SUBSTEP
+  };
+  for (int kt = 0; kt + 1 < nk; ++kt) {
+    if (kt + 2 < nk) request(kt + 2, ca);  // two steps ahead, into the register set decoded during the previous step
+    step(kt, std::true_type{});
+    {
+      const Codes tmp = ca;
+      ca = cb;
+      cb = tmp;
+    }
+    lds_sync();
+  }
+  step(nk - 1, std::false_type{});
+  lds_sync();
+  store_workgroup_tile<WN, WM, NWM>(p, acc, reinterpret_cast<uint8_t *>(sT), reinterpret_cast<uint8_t *>(sT + (BN + BM) * 8), m_base,
+                                    n_base, wave, lane);
+}
+
+template <int NWM>
+int launch_nvfp4_lds16(const GemmParams &p, hipStream_t st) {
+  const int total = ((p.M + 255) / 256 + (p.seg ? p.n_seg : 0)) * ((p.N + 255) / 256);
+  const int grid = ((total + 7) / 8) * 8;
+  hipLaunchKernelGGL(gemm_nvfp4_lds16<NWM>, dim3(grid), dim3(128 * NWM), 0, st, p);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+#endif  // ARCQ_EXPERIMENTS
+
 // ---------------------------------------------------------------------------------------------
 // Skinny kernels for M <= 64 (decode batches): the GEMM is a stream of the weight matrix, read
 // exactly once, so nothing is staged through LDS.  A workgroup owns 16 weight rows; its NW waves
@@ -1466,7 +1646,11 @@ GemmPlan plan_gemm(int M, int N, int Kp, int fmt, bool scales_aligned) {
     // against 74 us with 256x128 tiles), so the next smaller tile that still fills it
     const long t44 = (long)((M + 255) / 256) * ((N + 255) / 256), t42 = (long)((M + 127) / 128) * ((N + 255) / 256);
     const int pick = t44 >= 192 ? 44 : (M > 128 && !one_round_21 ? (t42 >= 192 ? 42 : 22) : 21);
-    const bool known = force == 44 || force == 84 || force == 42 || force == 22 || force == 21 || force == 11;
+#ifdef ARCQ_EXPERIMENTS
+    const bool known = force == 44 || force == 84 || force == 86 || force == 46 || force == 42 || force == 22 || force == 21 || force == 11;
+#else
+    const bool known = force == 44 || force == 42 || force == 22 || force == 21 || force == 11;
+#endif
     plan.kernel = known ? force : pick;  // a forced kernel that NVFP4 does not have is ignored
     return plan;
   }
@@ -1512,7 +1696,11 @@ int run_gemm(GemmParams p, const GemmPlan &plan, int fmt, float *scratch, hipStr
   } else {
     switch (plan.kernel) {
       case 44: return launch_nvfp4_tiled<4, 4>(p, st);
+#ifdef ARCQ_EXPERIMENTS
       case 84: return launch_nvfp4_tiled<4, 2, 4>(p, st);  // 256x256 tile, eight waves of 128x64
+      case 86: return launch_nvfp4_lds16<4>(p, st);       // 256x256 tile, operands decoded once per workgroup: eight waves,
+      case 46: return launch_nvfp4_lds16<2>(p, st);       // four waves
+#endif
       case 42: return launch_nvfp4_tiled<4, 2>(p, st);
       case 22: return launch_nvfp4_tiled<2, 2>(p, st);
       case 21: return launch_nvfp4_tiled<2, 1>(p, st);
