@@ -117,6 +117,10 @@ def probe_lib() -> ctypes.CDLL:
         P.arcq_stream_probe_variant.argtypes = [vp, vp, sz, sz, i, vp]
         P.arcq_stream_probe_variant.restype = i
         P.arcq_stream_probe_variants.restype = i
+        P.arcq_mfma_rate_probe.argtypes = [i, i, i, vp, vp, vp]
+        P.arcq_mfma_rate_probe.restype = i
+        P.arcq_mfma_rate_probe_flops.argtypes = [i, i, i]
+        P.arcq_mfma_rate_probe_flops.restype = ctypes.c_double
         _probe = P
     return _probe
 

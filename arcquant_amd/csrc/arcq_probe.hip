@@ -78,6 +78,60 @@ __global__ __launch_bounds__(1024) void stream_probe_lds_kernel(const v4u32 *src
   if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && n16_out) dst[0] = acc;
 }
 
+
+// Register-only matrix-pipe loops: what the MFMA units sustain with the operands the GEMMs feed them, with no
+// loads, LDS traffic or barriers.  Every wave keeps NACC independent 32x32 accumulators and four operand registers
+// per side, filled from `src` (4096 words: zeros, random bits, decoded-FP4-like fp16 values ...: the rate depends
+// on the data, the chip lowers its clock under the multipliers' switching power).  KIND 0: v_mfma_scale_f32_32x32x64_f8f6f4
+// with FP4 operands and E8M0 block scales (the MXFP4 GEMM's instruction), 1: v_mfma_f32_32x32x16_f16 (NVFP4's),
+// 2: v_mfma_f32_32x32x16_bf16 (the bf16 baseline's).
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+
+template <int KIND, int NACC>
+__global__ __launch_bounds__(512) void mfma_rate_kernel(const int *src, float *out, int iters) {
+  v8i a[4], b[4];
+  for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < 8; ++j) {
+      a[i][j] = src[(threadIdx.x * 8 + j + i * 17) & 4095];
+      b[i][j] = src[(threadIdx.x * 8 + j + i * 29 + 5) & 4095];
+    }
+  int sa[4], sb[4];
+  for (int i = 0; i < 4; ++i) {
+    sa[i] = (src[(threadIdx.x + i) & 4095] & 0x03030303) + 0x7e7e7e7e;  // E8M0 bytes near 2^0
+    sb[i] = (src[(threadIdx.x + 9 + i) & 4095] & 0x03030303) + 0x7e7e7e7e;
+  }
+  v16f acc[NACC];
+  for (int i = 0; i < NACC; ++i)
+    for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int i = 0; i < NACC; ++i) {
+        if (KIND == 0) {
+          acc[i] = ks == 0   ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i & 3], b[(i >> 2) & 3], acc[i], 4, 4, 0, sa[i & 3], 0, sb[(i >> 2) & 3])
+                   : ks == 1 ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i & 3], b[(i >> 2) & 3], acc[i], 4, 4, 1, sa[i & 3], 1, sb[(i >> 2) & 3])
+                   : ks == 2 ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i & 3], b[(i >> 2) & 3], acc[i], 4, 4, 2, sa[i & 3], 2, sb[(i >> 2) & 3])
+                             : __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i & 3], b[(i >> 2) & 3], acc[i], 4, 4, 3, sa[i & 3], 3, sb[(i >> 2) & 3]);
+        } else {
+          const v4i_t al = {a[i & 3][0], a[i & 3][1], a[i & 3][2], a[i & 3][3]}, bl = {b[(i >> 2) & 3][0], b[(i >> 2) & 3][1], b[(i >> 2) & 3][2], b[(i >> 2) & 3][3]};
+          if (KIND == 1)
+            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, al), __builtin_bit_cast(v8h, bl), acc[i], 0, 0, 0);
+          else
+            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, al), __builtin_bit_cast(v8bf, bl), acc[i], 0, 0, 0);
+        }
+      }
+  }
+  float s = 0;
+  for (int i = 0; i < NACC; ++i)
+    for (int v = 0; v < 16; ++v) s += acc[i][v];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 }  // namespace
 }  // namespace arcq
 
@@ -119,6 +173,29 @@ int arcq_stream_probe_variants(void) { return 11; }
 
 int arcq_stream_probe(const void *src, void *dst, size_t bytes_in, size_t bytes_out, void *stream) {
   return arcq_stream_probe_variant(src, dst, bytes_in, bytes_out, 0, stream);
+}
+
+
+int arcq_mfma_rate_probe(int kind, int waves_per_simd, int iters, const void *src, void *out, void *stream) {
+  if (!src || !out) return ARCQ_PROBE_ERR_NULL;
+  if (kind < 0 || kind > 2 || (waves_per_simd != 1 && waves_per_simd != 2) || iters < 1) return ARCQ_PROBE_ERR_SHAPE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int *s = static_cast<const int *>(src);
+  float *o = static_cast<float *>(out);
+  const dim3 grid(256), block(256 * waves_per_simd);  // one workgroup per CU
+#define ARCQ_RATE(K, NACC) hipLaunchKernelGGL((arcq::mfma_rate_kernel<K, NACC>), grid, block, 0, st, s, o, iters)
+  if (kind == 0) ARCQ_RATE(0, 8);  // eight independent accumulators per wave: half a wave's register file
+  else if (kind == 1) ARCQ_RATE(1, 8);
+  else ARCQ_RATE(2, 8);
+#undef ARCQ_RATE
+  return hipGetLastError() == hipSuccess ? ARCQ_PROBE_OK : ARCQ_PROBE_ERR_LAUNCH;
+}
+
+double arcq_mfma_rate_probe_flops(int kind, int waves_per_simd, int iters) {
+  // 256 CUs x 4 SIMDs x waves x iters x 4 sub-steps x accumulators x flops of one instruction
+  const double per_instr = kind == 0 ? 2.0 * 32 * 32 * 64 : 2.0 * 32 * 32 * 16;
+  const int nacc = 8;
+  return 256.0 * 4 * waves_per_simd * (double)iters * 4 * nacc * per_instr;
 }
 
 }  // extern "C"

@@ -118,6 +118,44 @@ def cpu_baseline(torch, sample_rows):
                       f"model/quantize.py fake_reorder_quantize_x after HF RMSNorm), best of {runs} runs, {best:.3f} s each"}
 
 
+def mfma_sustained(torch, iters=4000):
+    """What the matrix pipe sustains in a register-only loop (no loads, LDS or barriers) on all 256 CUs, by
+    instruction and by operand data: the chip lowers its clock under the multipliers' switching power, so the
+    ceiling for real operands is well below the data-sheet peak that roofline fractions are quoted against."""
+    import ctypes
+    from arcquant_amd import _lib
+    P = _lib.probe_lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    g = torch.Generator().manual_seed(11)
+    rnd = torch.randint(-2 ** 31, 2 ** 31 - 1, (4096,), generator=g, dtype=torch.int64).to(torch.int32)
+    # fp16 values as the NVFP4 decode produces them: an FP4 magnitude times (1 + m/8) * 2^e, random signs
+    mags = torch.tensor([0, .5, 1, 1.5, 2, 3, 4, 6])[torch.randint(0, 8, (8192,), generator=g)]
+    vals = mags * (1 + torch.randint(0, 8, (8192,), generator=g) / 8.0) * torch.pow(2.0, torch.randint(-3, 3, (8192,), generator=g).float())
+    vals = (vals * (torch.randint(0, 2, (8192,), generator=g) * 2 - 1)).to(torch.float16)
+    gauss = torch.randn(8192, generator=g).to(torch.bfloat16)
+    data = {"zeros": torch.zeros(4096, dtype=torch.int32), "random bits": rnd,
+            "decoded FP4 x E4M3 as fp16": vals.view(torch.int32), "N(0,1) as bf16": gauss.view(torch.int32)}
+    out = torch.empty(256 * 512, dtype=torch.float32, device="cuda")
+    rows = []
+    for kind, name, kinds_of_data in ((0, "v_mfma_scale_f32_32x32x64_f8f6f4 (FP4, E8M0 scales)", ("zeros", "random bits")),
+                                      (1, "v_mfma_f32_32x32x16_f16", ("zeros", "random bits", "decoded FP4 x E4M3 as fp16")),
+                                      (2, "v_mfma_f32_32x32x16_bf16", ("zeros", "random bits", "N(0,1) as bf16"))):
+        for dname in kinds_of_data:
+            src = data[dname].cuda()
+            for wps in (1, 2):
+                P.arcq_mfma_rate_probe(kind, wps, 50, src.data_ptr(), out.data_ptr(), stream)
+                torch.cuda.synchronize()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                P.arcq_mfma_rate_probe(kind, wps, iters, src.data_ptr(), out.data_ptr(), stream)
+                b.record()
+                torch.cuda.synchronize()
+                ms = a.elapsed_time(b)
+                rows.append({"instruction": name, "operands": dname, "waves_per_simd": wps,
+                             "tflops": round(P.arcq_mfma_rate_probe_flops(kind, wps, iters) / ms / 1e9, 1)})
+    return rows
+
+
 def gemm_rows(torch, agemm, shapes, Ms, fmts, iters=40):
     """ARC GEMM through the C ABI on preallocated outputs.  The quantized weights rotate over enough
     copies (> 300 MB) that every launch streams them from HBM, as a model's layers do; the bf16
@@ -381,6 +419,7 @@ def main():
     ap.add_argument("--gemm-ms", default="", help="M[,M...]: restrict the GEMM rows to these M")
     ap.add_argument("--no-layers", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    ap.add_argument("--mfma-probe", action="store_true", help="only the register-only matrix-pipe rates (one JSON line of its own)")
     ap.add_argument("--cpu-rows", type=int, default=M_TOKENS)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -397,6 +436,9 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     torch.cuda.set_device(0)
+    if args.mfma_probe:
+        print(json.dumps({"mfma_sustained": mfma_sustained(torch)}), flush=True)
+        return
     L = _lib.lib()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)   # launches and events share this stream
 
@@ -519,6 +561,38 @@ def main():
         name = {"x_unit": "reorder_quantize_x (tensor scale 1)", "x_scaled": "reorder_quantize_x (tensor scale max|x|/2688 on the device)"}[kind]
         quant.append({"op": name, "fmt": fmt, "select_num": S, "M": M_TOKENS, "us": round(ms * 1e3, 2),
                       "GB/s": round(b / ms / 1e6, 1), "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)})
+    if not args.no_quantize_table:
+        # what an NVFP4 linear's input costs in full (model/qLlamaLayer.py:73-77: the tensor scale, then the
+        # quantizer): arcq_tensor_scale + arcq_reorder_quantize_x with the scale read on the device, as one row
+        q, sf = outputs("NVFP4", SELECT)
+        sc = torch.empty((), dtype=torch.float32, device="cuda")
+
+        def scale_then_quantize(i):
+            L.arcq_tensor_scale(xs[i % nbuf].data_ptr(), None, H, M_TOKENS, H, 2688.0, sc.data_ptr(), stream)
+            L.arcq_reorder_quantize_x(xs[i % nbuf].data_ptr(), M_TOKENS, H, idx.data_ptr(), SELECT, fid["NVFP4"], 1.0,
+                                      ctypes.c_void_p(sc.data_ptr()), q.data_ptr(), sf.data_ptr(), stream)
+        ms_both = time_quant(scale_then_quantize, M_TOKENS, 100)
+        ms_scale = time_quant(lambda i: L.arcq_tensor_scale(xs[i % nbuf].data_ptr(), None, H, M_TOKENS, H, 2688.0,
+                                                            sc.data_ptr(), stream), M_TOKENS, 100)
+        b = quant_bytes(M_TOKENS, H, SELECT, "NVFP4", False) + 2 * M_TOKENS * H      # the tensor is read twice
+        quant.append({"op": "tensor_scale + reorder_quantize_x (two launches)", "fmt": "NVFP4", "select_num": SELECT, "M": M_TOKENS,
+                      "us": round(ms_both * 1e3, 2), "tensor_scale_us": round(ms_scale * 1e3, 2),
+                      "GB/s": round(b / ms_both / 1e6, 1), "frac_hbm": round(b / ms_both / 1e6 / HBM_PEAK_GBS, 4)})
+        # the fused norm at the prefill size of benchmark configuration 4 (16384 rows, rotating inputs): the rate
+        # without the ramp of a 13 us launch
+        M4 = 16384
+        x4 = [torch.cat([xs[(4 * j + k) % nbuf] for k in range(4)]) for j in range(max(2, nbuf // 4))]
+        for fmt in ("NVFP4", "MXFP4"):
+            q4, sf4 = outputs(fmt, SELECT, M4)
+            fn = lambda i, fmt=fmt, q4=q4, sf4=sf4: L.arcq_rmsnorm_quantize_x(
+                x4[i % len(x4)].data_ptr(), gam.data_ptr(), EPS, M4, H, idx.data_ptr(), SELECT, fid[fmt], 1.0, None,
+                q4.data_ptr(), sf4.data_ptr(), stream)
+            ms = time_quant(fn, M4, 50)
+            b = quant_bytes(M4, H, SELECT, fmt, True)
+            quant.append({"op": "rmsnorm_quantize_x", "fmt": fmt, "select_num": SELECT, "M": M4, "us": round(ms * 1e3, 2),
+                          "GB/s": round(b / ms / 1e6, 1), "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)})
+        del x4
+        torch.cuda.empty_cache()
     # long rows: the down projection's input at Llama-3-8B width (14336) and at the reference's widest dedicated
     # shape (28672, kernels/src/down.cu:71-233), 4096 rows each, tensor scale 1; rate per byte side by side
     if not args.no_quantize_table:
@@ -553,6 +627,17 @@ def main():
         out["gemm_peaks_tflops"] = MFMA_PEAK_TFLOPS
     if not (args.quick or args.no_layers):
         out["layers"] = layer_rows(torch)
+    if not args.quick:
+        out["mfma_sustained"] = mfma_sustained(torch)
+        # MoE routing (arcq_moe_route: two launches, three beyond 16384 tokens) by token count, 8 experts, top-2
+        route = []
+        for T in (4096, 16384, 32768, 65536):
+            lg = torch.randn(T, 8, device="cuda").to(torch.bfloat16)
+            for _ in range(3):
+                agemm.moe_route(lg, 2)
+            ms = loop_time_ms(lambda i: agemm.moe_route(lg, 2), 20, torch)
+            route.append({"tokens": T, "us": round(ms * 1e3, 1)})
+        out["moe_route"] = route
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, args.cpu_rows)

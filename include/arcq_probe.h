@@ -31,6 +31,19 @@ int arcq_stream_probe(const void *src, void *dst, size_t bytes_in, size_t bytes_
 int arcq_stream_probe_variant(const void *src, void *dst, size_t bytes_in, size_t bytes_out, int variant, void *stream);
 int arcq_stream_probe_variants(void);
 
+/*
+ * Register-only matrix-pipe loop on all 256 CUs (one workgroup per CU, waves_per_simd = 1 or 2 waves on every
+ * SIMD): what the MFMA units sustain on given operand bits without loads, LDS traffic or barriers.
+ *   kind  0: v_mfma_scale_f32_32x32x64_f8f6f4 on FP4 operands with E8M0 block scales (the MXFP4 GEMM's instruction)
+ *         1: v_mfma_f32_32x32x16_f16 (what NVFP4 decodes to), 2: v_mfma_f32_32x32x16_bf16 (the bf16 baseline)
+ *   src   4096 32-bit words on the device that fill the operand registers: the sustained rate depends on them
+ *         (zeros, random bits, fp16 values with three mantissa bits ...), the chip lowers its clock under load
+ *   out   256 * 512 floats on the device (keeps the arithmetic alive)
+ * arcq_mfma_rate_probe_flops: floating-point operations one such launch performs.
+ */
+int arcq_mfma_rate_probe(int kind, int waves_per_simd, int iters, const void *src, void *out, void *stream);
+double arcq_mfma_rate_probe_flops(int kind, int waves_per_simd, int iters);
+
 #ifdef __cplusplus
 }
 #endif

@@ -136,6 +136,10 @@ def test_probe_library_is_separate_from_the_product_library():
     """the copy kernels used for measurement live in their own library with their own header"""
     P, L = _lib.probe_lib(), _lib.lib()
     names = declared_symbols("arcq_probe.h")
-    assert names == ["arcq_stream_probe", "arcq_stream_probe_variant", "arcq_stream_probe_variants"]
+    assert names == ["arcq_mfma_rate_probe", "arcq_mfma_rate_probe_flops", "arcq_stream_probe", "arcq_stream_probe_variant",
+                     "arcq_stream_probe_variants"]
+    assert P.arcq_mfma_rate_probe(3, 1, 10, ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1000), None) == 2
+    assert P.arcq_mfma_rate_probe_flops(0, 2, 1) == 256.0 * 4 * 2 * 4 * 8 * 2.0 * 32 * 32 * 64
+    assert P.arcq_mfma_rate_probe_flops(1, 1, 3) == 256.0 * 4 * 1 * 3 * 4 * 8 * 2.0 * 32 * 32 * 16
     for n in names:
         assert hasattr(P, n) and not hasattr(L, n)
