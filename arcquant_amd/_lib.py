@@ -58,6 +58,7 @@ def lib() -> ctypes.CDLL:
     L.arcq_swiglu_quantize_x.argtypes = [vp, vp, i, i, i, vp, i, i, f, vp, vp, vp, vp]
     L.arcq_swiglu_absmax.argtypes = [vp, vp, i, i, i, vp, vp]
     L.arcq_tensor_scale.argtypes = [vp, vp, i, i, i, f, vp, vp]
+    L.arcq_reorder_quantize_x_absmax.argtypes = [vp, i, i, vp, i, i, f, vp, vp, vp, vp]
     L.arcq_kv_append_i4.argtypes = [vp, vp, i, i, vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
     L.arcq_rope_kv_append_i4.argtypes = [vp, i, i, i, i, vp, vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
     L.arcq_rope.argtypes = [vp, i, i, ctypes.c_long, i, i, i, i, i, vp, vp, i, vp, vp, vp]

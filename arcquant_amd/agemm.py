@@ -93,9 +93,18 @@ def _quantize(entry, X, gamma, eps, reorder_index, KE, fmt, global_scale):
     if K % 32 or K < 32 or K > 32736 or KE < 0 or KE > K or KE % G:
         raise RuntimeError(f"Value error in {entry}: K={K}, KE={KE} not supported for {fmt} "
                            f"(need K % 32 == 0, 32 <= K <= 32736, KE % {G} == 0, KE <= K)")
-    gs, d_gs, keep = _scalar(global_scale, X.device)
     QX = torch.empty((M, (K + KE) // 2), dtype=torch.uint8, device=X.device)
     SFX = torch.empty((M * ((K + KE) // G),), dtype=torch.uint8, device=X.device)
+    if isinstance(global_scale, str):
+        if global_scale != "absmax" or entry != "arcq_reorder_quantize_x":
+            raise RuntimeError("global_scale must be a number or a tensor (reorder_quantize_x also takes 'absmax')")
+        scale = torch.empty((), dtype=torch.float32, device=X.device)
+        with _on_device(X):
+            rc = L.arcq_reorder_quantize_x_absmax(X.data_ptr(), M, K, reorder_index.data_ptr(), KE, f, 2688.0, scale.data_ptr(),
+                                                  QX.data_ptr(), SFX.data_ptr(), _stream(X))
+        _lib.check(rc, "arcq_reorder_quantize_x_absmax")
+        return QX, SFX, scale
+    gs, d_gs, keep = _scalar(global_scale, X.device)
     with _on_device(X):
         if gamma is None:
             rc = getattr(L, entry)(X.data_ptr(), M, K, reorder_index.data_ptr(), KE, f, gs, d_gs, QX.data_ptr(),
@@ -114,7 +123,10 @@ def _quantize(entry, X, gamma, eps, reorder_index, KE, fmt, global_scale):
 
 def reorder_quantize_x(X, reorder_index, KE, *, fmt="NVFP4", global_scale=None):
     """agemm.reorder_quantize_x (kernels/src/bindings.cpp:122-163).
-    X bf16 [M,K]; reorder_index int16 [K]; returns QX u8 [M,(K+KE)/2], SFX u8 [M*(K+KE)/G]."""
+    X bf16 [M,K]; reorder_index int16 [K]; returns QX u8 [M,(K+KE)/2], SFX u8 [M*(K+KE)/G].
+    global_scale="absmax" forms the NVFP4 tensor scale max|X| / 2688 on the device as part of the call (what the
+    reference's callers compute with torch first, model/qLlamaLayer.py:73-77) and returns it as a third value:
+    one launch and one pass over X while X fits the chip's LDS (up to 4096 rows of up to 4096 channels)."""
     return _quantize("arcq_reorder_quantize_x", X, None, 0.0, reorder_index, KE, fmt, global_scale)
 
 

@@ -3,6 +3,7 @@
     python -m arcquant_amd.build            # build if stale
     python -m arcquant_amd.build --force    # rebuild even if up to date
     python -m arcquant_amd.build --experiments   # with the measured-and-not-taken kernel variants (ARCQ_GEMM_KERNEL)
+    python -m arcquant_amd.build --phases KERNEL # instruction counts between the ARCQ_PHASE markers of one kernel
 
 hipcc cross-compiles for gfx950 without a GPU present.  The built libraries live next to the
 sources (arcquant_amd/csrc/) so that they travel with the tree.
@@ -74,5 +75,59 @@ def build_all(force: bool = False, verbose: bool = False, experiments: bool = Fa
     return (build_hip(force or experiments, verbose, experiments), build_probe(force, verbose))
 
 
+def phase_listing(kernel: str, source: str = "arcq_quantize.hip") -> str:
+    """Static instruction counts of one kernel, cut at its ARCQ_PHASE markers and at every label, in the order of
+    the compiler's assembly (the device pass alone, -S, with -DARCQ_PHASE_MARKERS: the markers are comments, the
+    code is the normal build's).  `kernel` is a substring of the mangled name.  Which pieces run how often per row
+    follows from the branches, which the listing shows with their targets."""
+    import re
+    import tempfile
+    flags = [f for f in HIPCC_FLAGS if f not in ("-fPIC", "-shared")]
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "k.s")
+        subprocess.check_call([_hipcc(), *flags, "-DARCQ_PHASE_MARKERS", "--cuda-device-only", "-S", "-o", out,
+                               os.path.join(CSRC, source)], stderr=subprocess.DEVNULL)
+        text = open(out).read()
+    m = re.search(r"^(\S*%s\S*):" % re.escape(kernel), text, re.M)
+    if not m:
+        raise SystemExit(f"no kernel matching {kernel!r} in {source}")
+    body = text[m.end():text.index(".Lfunc_end", m.end())].split("\n")
+    classes = ("valu", "salu", "lds", "vmem")
+    rows, phase, label, cur, notes = [], "entry", "", dict.fromkeys(classes, 0), []
+
+    def flush():
+        if any(cur.values()) or notes:
+            rows.append((label, phase, dict(cur), " ".join(notes)))
+        for c in classes:
+            cur[c] = 0
+        notes.clear()
+
+    for line in body:
+        mark = re.search(r"; ARCQ_PHASE (.*)", line)
+        lab = re.match(r"(\.LBB\w+):", line)
+        if mark or lab:
+            flush()
+            if mark:
+                phase = mark.group(1).strip()
+            else:
+                label = lab.group(1)
+            continue
+        w = line.split()
+        if not line.startswith("\t") or not w or w[0][0] in ".;":
+            continue
+        op = w[0]
+        cur["valu" if op.startswith("v_") else "salu" if op.startswith("s_") else "lds" if op.startswith("ds_") else "vmem"] += 1
+        if op.startswith(("s_cbranch", "s_branch")):
+            notes.append(f"{op[2:]}->{w[1]}")
+    flush()
+    lines = [f"{m.group(1)}", f"{'label':10s} {'phase':42s} {'VALU':>5s} {'SALU':>5s} {'LDS':>4s} {'VMEM':>5s}  branches"]
+    for lab, ph, c, n in rows:
+        lines.append(f"{lab:10s} {ph:42s} {c['valu']:5d} {c['salu']:5d} {c['lds']:4d} {c['vmem']:5d}  {n}")
+    return "\n".join(lines)
+
+
 if __name__ == "__main__":
+    if "--phases" in sys.argv:
+        print(phase_listing(sys.argv[sys.argv.index("--phases") + 1]))
+        sys.exit(0)
     print(build_all(force="--force" in sys.argv, verbose=True, experiments="--experiments" in sys.argv))

@@ -96,6 +96,7 @@ const Tuning &tuning() {
     if (const char *e = getenv("ARCQ_QUANT_GRID")) v.quant_grid = atoi(e);
     if (const char *e = getenv("ARCQ_QUANT_KERNEL")) v.quant_kernel = atoi(e);
     if (const char *e = getenv("ARCQ_KV_DECODE_SPLITS")) v.kv_decode_splits = atoi(e);
+    if (const char *e = getenv("ARCQ_RESIDENT_SPIN_US")) v.resident_spin_us = atoi(e);
     return v;
   }();
   return t;

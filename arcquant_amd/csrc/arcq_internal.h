@@ -25,12 +25,13 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 // kept until the process ends, so that a captured graph may hold its address.  Work on one stream is
 // serialised, so two calls never share a buffer unless they share a stream.
 enum WorkspaceKind {
-  kWsTensorScale = 0,  // (maximum, arrival counter) pairs of arcq_tensor_scale, one per 128-byte line (zeroed once)
+  kWsTensorScale = 0,  // (maximum, arrival counter) pairs of arcq_tensor_scale, one per 128-byte line, and from byte 2048
+                       // the workgroups' slots of the one-launch scale + quantizer (zeroed once)
   kWsSplitK = 1,       // fp32 partial tiles of the split-K GEMM
   kWsDecode = 2,       // partial softmax sums of the split decode attention
   kWsKinds = 3
 };
-constexpr size_t kWorkspaceBytes[kWsKinds] = {2048, 32u << 20, 8u << 20};
+constexpr size_t kWorkspaceBytes[kWsKinds] = {4096, 32u << 20, 8u << 20};
 
 // The buffer of `kind` for (current device, stream).  Returns nullptr and sets *status when there is
 // none and none can be made: ARCQ_ERR_WORKSPACE while `stream` is capturing (an allocation there
@@ -56,6 +57,8 @@ int noalloc_prepare();
 //   ARCQ_QUANT_KERNEL=<1|2|3>   1 = never, 2 = always take the wave-per-row quantizer where it has an instance;
 //                               3 = the four-units-per-thread kernel of the rows beyond 16384 channels from 1024 channels on
 //   ARCQ_KV_DECODE_SPLITS=<n>   ranges per sequence of the decode attention
+//   ARCQ_RESIDENT_SPIN_US=<n>   how long a workgroup of the one-launch scale + quantizer waits for the others before it takes
+//                               the tensor's maximum by itself (0: at once; -1: always two launches instead)
 // Unset (the normal case) every field keeps the value below and the dispatch is the measured one.
 struct Tuning {
   int gemm_kernel = -1;
@@ -64,6 +67,7 @@ struct Tuning {
   int quant_grid = 0;
   int quant_kernel = 0;
   int kv_decode_splits = 0;
+  int resident_spin_us = 200;
 };
 const Tuning &tuning();
 

@@ -846,6 +846,14 @@ __global__ __launch_bounds__(512, 4) void quantize_rows_wide_kernel(QuantParams 
 // ---------------------------------------------------------------------------------------------
 constexpr int kRowWaves = 16;  // waves per workgroup = rows in progress per CU (four per SIMD)
 
+// Comment-only markers in the compiler's assembly output (-DARCQ_PHASE_MARKERS), for counting the instructions of
+// each phase of the wave-per-row kernel; nothing in a normal build.
+#ifdef ARCQ_PHASE_MARKERS
+#define ARCQ_PHASE(name) asm volatile("; ARCQ_PHASE " name)
+#else
+#define ARCQ_PHASE(name)
+#endif
+
 template <int OFF>
 __device__ __forceinline__ void row_dma16(const void *g, uint32_t lds_base) {
   // writes M0 (reserved: cannot be listed as clobbered); nothing else in this kernel reads M0
@@ -946,6 +954,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_wave_kernel(Quan
     wait_vm<0>();  // the row has landed (past the first row this also waits for the previous row's stores;
                    // the SIMD's other waves fill the gap)
     if (MODE == MODE_NORM) {
+      ARCQ_PHASE("pass1 sum of squares");
       // pass 1 over the lane's natural-order values: sum of squares (exact squares, fp64 accumulation)
       double ss0 = 0.0, ss1 = 0.0;
 #pragma unroll
@@ -959,6 +968,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_wave_kernel(Quan
           ss1 = __builtin_fma(d1, d1, ss1);
         }
       }
+      ARCQ_PHASE("wave reduction and 1/sqrt");
       double tot = wave_sum_to_lane63(ss0 + ss1);
       {
         const uint64_t b = __builtin_bit_cast(uint64_t, tot);
@@ -977,6 +987,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_wave_kernel(Quan
       } else {
         rstd = 1.0f / sqrtf(a);
       }
+      ARCQ_PHASE("pass2 normalise and gamma");
       // pass 2: normalise, multiply by gamma, write the bf16 results over the raw values this lane read
       const uint4 *glo_t = reinterpret_cast<const uint4 *>(lds + SLOT), *ghi_t = reinterpret_cast<const uint4 *>(lds + 2 * SLOT);
 #pragma unroll
@@ -994,6 +1005,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_wave_kernel(Quan
       // the gather below reads what other lanes wrote: LDS operations of one wave execute in order
     }
 
+    ARCQ_PHASE("units: gather addresses, encode, stores");
     uint8_t *crow = p.codes + (size_t)row * (Kp >> 1), *srow = p.scales + (size_t)row * (Kp / G);
     const int next_row = row + stride;
     {
@@ -1028,6 +1040,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_wave_kernel(Quan
       const int n = u * 64 + lane;
       store_unit<FMT>(crow, srow, n, pk, sb);
       if (u * 64 + 63 >= tail0) {  // wave-uniform: some lane's unit of this round is among the last select_num channels
+        ARCQ_PHASE("residual block");
         float e[16];
         decode_unit(pk, e);
 #pragma unroll
@@ -1037,10 +1050,249 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_wave_kernel(Quan
         const uint32_t sb2 = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t2, &s2) : ue8m0_scale(t2, &s2);
         const uint2 pk2 = encode_unit_coarse(e, scale_rcp<FMT>(s2));
         if (n >= tail0) store_unit<FMT>(crow, srow, nunits + (n - tail0), pk2, sb2);
+        ARCQ_PHASE("units (continued)");
       }
     }
+    ARCQ_PHASE("row loop end");
     if (next_row >= p.rows) break;
     row = next_row;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tensor scale and quantizer in one launch, for activations that fit the chip's LDS (sixteen rows of up to 4096
+// channels per CU: 4096 rows on 256 CUs).  The reference's callers form max|x| / 2688 with torch ahead of the
+// quantizer (model/qLlamaLayer.py:73-77): two passes over x.  Here a wave loads its row into LDS once, the
+// workgroups exchange their maxima, and the rows are encoded from LDS under the scale.
+//
+// Exchange: workgroup b stores (tag, maximum) as one 64-bit word into slot b; wave 0 of every workgroup reads all
+// slots until each carries the launch's tag.  The tag is one more than the value of an epoch word read at the
+// start; on its way out every workgroup raises the epoch word to its tag (atomic maximum), so the next launch on
+// the stream -- which starts after this one has ended -- takes a tag above every tag ever stored.  No counter to
+// reset, no read-modify-write on the way in, nothing the host has to pass: a captured launch replays correctly.
+//
+// The workgroups can only meet if all of them are on the chip at once, which nothing guarantees (another kernel
+// may hold CUs).  So the wait is bounded: when it runs out the workgroup takes the maximum over the whole tensor
+// by itself, from global memory, and goes on.  Every workgroup therefore finishes whatever the others do; the
+// result is the same either way (a maximum), the bounded wait only decides how it was obtained.
+// ---------------------------------------------------------------------------------------------
+constexpr int kResidentSlots = 256;        // workgroups per launch at most (512 of half the size: 2 us slower at 2048 rows)
+constexpr int kResidentSlotWord = 256;     // slots start at this 64-bit word of the tensor-scale scratch (byte 2048)
+constexpr int kResidentEpochWord = 480;   // 32-bit word of the epoch, on a 128-byte line of its own behind the
+                                          // (maximum, counter) pairs of tensor_scale_kernel
+
+typedef uint16_t v2u16 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t absmax_bf16_pairs(uint32_t m, uint32_t w) {
+  const v2u16 a = __builtin_bit_cast(v2u16, m), b = __builtin_bit_cast(v2u16, w & 0x7fff7fffu);
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));  // v_pk_max_u16
+}
+
+// WPR waves share a row (1, 2 or 4: a row's units are dealt out to them by whole rounds of 64), so that a launch of
+// few rows still spreads over the chip: a workgroup holds 16 / WPR rows, and a wave's share of the arithmetic that
+// follows the exchange -- where nothing else can hide it -- is 1 / WPR of a row.
+template <int FMT, int KU, int WPR>
+__global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(QuantParams p, float divisor, uint32_t spin_ticks,
+                                                                                 uint32_t *ws, float *scale_out) {
+  extern __shared__ uint4 smem[];
+  constexpr int G = FMT == ARCQ_FMT_NVFP4 ? 16 : 32;
+  constexpr int K = 1024 * KU, NCH = 2 * KU, SLOT = 2 * K;
+  constexpr int TABLES = SLOT;  // reorder_index
+  constexpr int RPW = kRowWaves / WPR;  // rows per workgroup
+  constexpr int UPL = KU / WPR;         // units per lane
+  constexpr int CPW = NCH / WPR;        // 1024-byte chunks of the row that a wave fetches
+  static_assert(KU % WPR == 0 && kRowWaves % WPR == 0, "a row's rounds of 64 units are dealt out whole");
+  const int S = p.S, Kp = K + S;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r_in = wave / WPR;
+  // which part of the row: rotated from row to row, so that the waves that own the last select_num channels (and
+  // encode the residual on top) fall on different SIMDs (wave i of a workgroup runs on SIMD i mod 4)
+  const int sub = WPR == 1 ? 0 : (wave + r_in) % WPR;
+  uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
+  const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>(lds);
+  const uint32_t slot_addr = lds0 + TABLES + r_in * SLOT;  // this wave's row
+  const uint4 *part = reinterpret_cast<const uint4 *>(lds + TABLES + r_in * SLOT + sub * CPW * 1024);
+  uint32_t *meet = reinterpret_cast<uint32_t *>(lds + TABLES + RPW * SLOT);  // [0..15] wave maxima, [16] maximum, [17] timed out
+  const int nunits = K >> 4, tail0 = (K - S) >> 4;
+  const int row = blockIdx.x * RPW + r_in;
+  const bool has_row = row < p.rows;
+  unsigned long long *slots = reinterpret_cast<unsigned long long *>(ws) + kResidentSlotWord;
+  uint32_t *epoch = ws + kResidentEpochWord;
+  const uint16_t *src = p.x + (size_t)row * K + sub * CPW * 512;
+  const uint32_t dst = slot_addr + sub * CPW * 1024;
+
+  // rows and table as in the wave-per-row kernel above: four waves request their rows ahead of the table
+  constexpr int kEarlyWaves = 4;
+  const bool early = wave >= kRowWaves - kEarlyWaves && has_row;
+  if (early) row_dma<CPW>(src, lane, dst);
+  if (wave < NCH) {
+    const uint8_t *g = reinterpret_cast<const uint8_t *>(p.idx) + 1024 * wave + 16 * lane;
+    row_dma16<0>(g, lds0 + 1024 * wave);
+  }
+  uint32_t tag = 0u;
+  if (wave == 0) tag = __hip_atomic_load(epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;  // every lane: uniform
+  if (early) wait_vm<CPW>();
+  else wait_vm<0>();
+  lds_barrier();
+  if (!early && has_row) row_dma<CPW>(src, lane, dst);
+  wait_vm<0>();
+
+  // what does not depend on the scale: the maximum, and the units' values in the channel order
+  uint32_t m = 0u;
+  uint32_t yp[UPL][8];
+#pragma unroll
+  for (int u = 0; u < UPL; ++u)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) yp[u][j] = 0u;
+  if (has_row) {
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      const uint4 q = part[c * 64 + lane];
+      m = absmax_bf16_pairs(absmax_bf16_pairs(absmax_bf16_pairs(absmax_bf16_pairs(m, q.x), q.y), q.z), q.w);
+    }
+  }
+  // A 16-bit LDS load into one half of a register clears the other half on this chip, so two channels cannot be
+  // loaded into one register: sixteen registers per unit (high halves), then one byte permute per pair.
+  auto gather_units = [&]() {
+    if (!has_row) return;
+    const uint4 *idx_t = reinterpret_cast<const uint4 *>(lds);
+    uint32_t ta[16], tb[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) ta[i] = tb[i] = 0u;
+    auto request = [&](int u, uint32_t (&t)[16]) {
+      const int n = (sub * UPL + u) * 64 + lane;
+      const uint4 i0 = idx_t[2 * n], i1 = idx_t[2 * n + 1];
+      const uint32_t iw[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
+      uint32_t addr[16];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        addr[2 * j] = gather_addr<0>(iw[j], slot_addr);
+        addr[2 * j + 1] = gather_addr<1>(iw[j], slot_addr);
+      }
+      gather16(t, addr);
+    };
+    request(0, ta);
+#pragma unroll
+    for (int u = 0; u < UPL; ++u) {
+      uint32_t(&cur)[16] = (u & 1) ? tb : ta;
+      uint32_t(&nxt)[16] = (u & 1) ? ta : tb;
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(cur[i]));  // read after the wait above
+#pragma unroll
+      for (int j = 0; j < 8; ++j) yp[u][j] = __builtin_amdgcn_perm(cur[2 * j + 1], cur[2 * j], 0x07060302u);
+      if (u + 1 < UPL) request(u + 1, nxt);
+    }
+  };
+  if (WPR == 1) gather_units();  // the row is this wave's own: no need to wait for anybody
+  m = (m & 0xffffu) > (m >> 16) ? (m << 16) : (m & 0xffff0000u);  // the larger half, as the bits of an fp32
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint32_t v = (uint32_t)__shfl_xor((int)m, o);
+    m = v > m ? v : m;
+  }
+  if (lane == 0) meet[wave] = m;
+  lds_barrier();  // the maxima are in LDS; every part of every row has landed
+
+  if (wave == 0) {
+    uint32_t wg = lane < kRowWaves ? meet[lane] : 0u;
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) {
+      const uint32_t v = (uint32_t)__shfl_xor((int)wg, o);
+      wg = v > wg ? v : wg;
+    }
+    wg = __builtin_amdgcn_readfirstlane(wg);
+    if (lane == 0)
+      __hip_atomic_store(slots + blockIdx.x, ((unsigned long long)tag << 32) | wg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (WPR != 1) gather_units();  // while the slot is on its way
+  if (wave == 0) {
+    // lane l watches slots l, l + 64, l + 128, ...
+    const int nslots = (int)gridDim.x;
+    uint32_t all = 0u;
+    unsigned pending = 0u;
+#pragma unroll
+    for (int j = 0; j < kResidentSlots / 64; ++j)
+      if (lane + 64 * j < nslots) pending |= 1u << j;
+    const unsigned long long t0 = wall_clock64();
+    bool timed_out = false;
+    for (;;) {
+#pragma unroll
+      for (int j = 0; j < kResidentSlots / 64; ++j) {
+        if (pending & (1u << j)) {
+          const unsigned long long v = __hip_atomic_load(slots + lane + 64 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if ((uint32_t)(v >> 32) == tag) {
+            const uint32_t mv = (uint32_t)v;
+            all = mv > all ? mv : all;
+            pending &= ~(1u << j);
+          }
+        }
+      }
+      if (__builtin_amdgcn_ballot_w64(pending != 0u) == 0ull) break;
+      if (wall_clock64() - t0 >= (unsigned long long)spin_ticks) {  // the clock is read once per wave
+        timed_out = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t v = (uint32_t)__shfl_xor((int)all, o);
+      all = v > all ? v : all;
+    }
+    if (lane == 0) {
+      meet[16] = all;
+      meet[17] = timed_out ? 1u : 0u;
+    }
+  }
+  lds_barrier();
+  uint32_t all = meet[16];
+  if (meet[17] != 0u) {
+    // the others did not show up in time: this workgroup takes the maximum over the whole tensor by itself
+    const size_t total = (size_t)p.rows * (K >> 3);
+    uint32_t mm = 0u;
+    for (size_t c = threadIdx.x; c < total; c += 64 * kRowWaves) {
+      const uint4 q = reinterpret_cast<const uint4 *>(p.x)[c];
+      mm = absmax_bf16_pairs(absmax_bf16_pairs(absmax_bf16_pairs(absmax_bf16_pairs(mm, q.x), q.y), q.z), q.w);
+    }
+    mm = (mm & 0xffffu) > (mm >> 16) ? (mm << 16) : (mm & 0xffff0000u);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t v = (uint32_t)__shfl_xor((int)mm, o);
+      mm = v > mm ? v : mm;
+    }
+    lds_barrier();  // meet[16], meet[17] have been read by everybody
+    if (lane == 0) meet[wave] = mm;
+    lds_barrier();
+    all = 0u;
+    for (int w = 0; w < kRowWaves; ++w) all = meet[w] > all ? meet[w] : all;
+  }
+  if (threadIdx.x == 0) atomicMax(epoch, tag);  // nobody waits for it: the next launch on the stream reads it
+  const float quot = u2f(all) / divisor;
+  const float g = quot == 0.0f ? 1.0f : quot;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = g;
+  if (!has_row) return;
+
+  const float rg = 1.0f / g;
+  const bool g_odd = !(fabsf(g) >= 0x1p-60f && fabsf(g) <= 0x1p+60f);
+  const bool coarse = (f2u(g) & 0x7fffffu) == 0u;
+  uint8_t *crow = p.codes + (size_t)row * (Kp >> 1), *srow = p.scales + (size_t)row * (Kp / G);
+#pragma unroll
+  for (int u = 0; u < UPL; ++u) {
+    uint32_t yv[16];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      yv[2 * j] = yp[u][j] << 16;
+      yv[2 * j + 1] = yp[u][j] & 0xffff0000u;
+    }
+    const int n = (sub * UPL + u) * 64 + lane;
+    const bool tail = n >= tail0;
+    uint2 pk, pk2;
+    uint32_t sb, sb2;
+    quantize_unit<FMT, MODE_X, true>(yv, true, tail, g, rg, g_odd, coarse, pk, sb, pk2, sb2);
+    store_unit<FMT>(crow, srow, n, pk, sb);
+    if (tail) store_unit<FMT>(crow, srow, nunits + (n - tail0), pk2, sb2);
   }
 }
 
@@ -1318,6 +1570,52 @@ int launch_quantize_wave_for(int fmt, int mode, const QuantParams &p, hipStream_
   ARCQ_WAVE_CASE(3)
   ARCQ_WAVE_CASE(4)
 #undef ARCQ_WAVE_CASE
+  return -1;
+}
+
+// tensor scale and quantizer in one launch (quantize_rows_resident_kernel); -1 when the tensor does not fit it
+template <int KU, int WPR>
+int launch_quantize_resident_as(const QuantParams &p, float divisor, float *d_scale, uint32_t *ws, hipStream_t st) {
+  constexpr int RPW = kRowWaves / WPR;
+  const size_t lds = (size_t)p.K * 2 * (1 + RPW) + 128;
+  const int grid = (p.rows + RPW - 1) / RPW;
+  const int spin_us = tuning().resident_spin_us;
+  const uint32_t ticks = (uint32_t)(spin_us < 0 ? 0 : spin_us) * 100u;  // the wall clock counts at 100 MHz
+  auto kern = quantize_rows_resident_kernel<ARCQ_FMT_NVFP4, KU, WPR>;
+  if (lds > 64 * 1024)
+    ARCQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kRowWaves), lds, st, p, divisor, ticks, ws, d_scale);
+  ARCQ_HIP_TRY(hipGetLastError());
+  return ARCQ_OK;
+}
+
+int launch_quantize_resident(const QuantParams &p, float divisor, float *d_scale, hipStream_t st) {
+  if (p.K % 1024 != 0 || p.K > 4096) return -1;
+  // As many waves per row as the rows leave room for: the workgroups must fit the chip all at once (160 KB of LDS
+  // per CU, 256 CUs) and the slots they meet on.
+  auto fits = [&](int wpr) {
+    const int rpw = kRowWaves / wpr;
+    const size_t lds = (size_t)p.K * 2 * (1 + rpw) + 128;
+    const int grid = (p.rows + rpw - 1) / rpw;
+    return grid <= kResidentSlots && grid <= 256 * (int)((160 * 1024) / lds);
+  };
+  const int ku = p.K >> 10;
+  int wpr = 0;
+  for (int w : {4, 2, 1})
+    if (wpr == 0 && ku % w == 0 && fits(w)) wpr = w;
+  if (wpr == 0) return -1;
+  int status = ARCQ_OK;
+  uint32_t *ws = static_cast<uint32_t *>(stream_workspace(kWsTensorScale, st, &status));
+  if (!ws) return status;
+  switch (ku * 10 + wpr) {
+    case 11: return launch_quantize_resident_as<1, 1>(p, divisor, d_scale, ws, st);
+    case 21: return launch_quantize_resident_as<2, 1>(p, divisor, d_scale, ws, st);
+    case 22: return launch_quantize_resident_as<2, 2>(p, divisor, d_scale, ws, st);
+    case 31: return launch_quantize_resident_as<3, 1>(p, divisor, d_scale, ws, st);
+    case 41: return launch_quantize_resident_as<4, 1>(p, divisor, d_scale, ws, st);
+    case 42: return launch_quantize_resident_as<4, 2>(p, divisor, d_scale, ws, st);
+    case 44: return launch_quantize_resident_as<4, 4>(p, divisor, d_scale, ws, st);
+  }
   return -1;
 }
 
@@ -1640,6 +1938,41 @@ int arcq_tensor_scale(const void *x, const void *up, int ld, int M, int K, float
                        d_scale);
   ARCQ_HIP_TRY(hipGetLastError());
   return ARCQ_OK;
+}
+
+int arcq_reorder_quantize_x_absmax(const void *x, int M, int K, const int16_t *reorder_index, int select_num, int fmt,
+                                   float divisor, float *d_scale, void *codes, void *scales, void *stream) {
+  if (fmt != ARCQ_FMT_NVFP4 && fmt != ARCQ_FMT_MXFP4) return ARCQ_ERR_FORMAT;
+  const int G = arcq_group_size(fmt);
+  if (M < 0 || K < 32 || K % 32 != 0 || K > 32736 || select_num < 0 || select_num > K || select_num % G != 0 || !(divisor > 0.0f))
+    return ARCQ_ERR_SHAPE;
+  if (!d_scale || (M > 0 && (!x || !reorder_index || !codes || !scales))) return ARCQ_ERR_NULL;
+  if (M > 0 && (!arcq::aligned16(x) || !arcq::aligned16(reorder_index) || !arcq::aligned16(codes))) return ARCQ_ERR_ALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (M > 0 && fmt == ARCQ_FMT_NVFP4 && arcq::tuning().resident_spin_us >= 0) {
+    arcq::QuantParams p;
+    p.x = static_cast<const uint16_t *>(x);
+    p.gamma = nullptr;
+    p.up = nullptr;
+    p.ldx = K;
+    p.idx = reorder_index;
+    p.codes = static_cast<uint8_t *>(codes);
+    p.scales = static_cast<uint8_t *>(scales);
+    p.d_gscale = nullptr;
+    p.gscale = 1.0f;
+    p.eps = 0.0f;
+    p.rows = M;
+    p.K = K;
+    p.S = select_num;
+    p.inv_k = 1.0 / (double)K;
+    const int rc = arcq::launch_quantize_resident(p, divisor, d_scale, st);
+    if (rc >= 0) return rc;
+  }
+  // tensors beyond the chip's LDS, other row lengths, MXFP4: the scale, then the quantizer under it
+  const int rc = arcq_tensor_scale(x ? x : d_scale, nullptr, K, M, K, divisor, d_scale, stream);
+  if (rc != ARCQ_OK) return rc;
+  return arcq::quantize_entry(arcq::MODE_X, x, nullptr, 0.0f, M, K, reorder_index, select_num, fmt, 1.0f, d_scale, codes, scales,
+                              stream);
 }
 
 int arcq_grouped_reorder_quantize_x(const void *x, int M, int K, const int *seg_offsets, int n_seg,

@@ -57,6 +57,9 @@ def _tensor_scale(t: torch.Tensor, signed: bool) -> torch.Tensor:
 def reorder_quantize_x(x, reorder_index, select_num, quant_type="NVFP4"):
     """model/qLlamaLayer.py:79-86: x bf16 [tokens, K] -> (qx, scale_x, scale)."""
     if quant_type == "NVFP4":
+        if x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.is_contiguous():
+            # scale and quantizer as one call: one launch and one pass over x while it fits the chip's LDS
+            return agemm.reorder_quantize_x(x, reorder_index, select_num, fmt="NVFP4", global_scale="absmax")
         scale = _tensor_scale(x, signed=False)
         qx, scale_x = agemm.reorder_quantize_x(x, reorder_index, select_num, fmt="NVFP4", global_scale=scale)
         return qx, scale_x, scale

@@ -578,6 +578,14 @@ def main():
         quant.append({"op": "tensor_scale + reorder_quantize_x (two launches)", "fmt": "NVFP4", "select_num": SELECT, "M": M_TOKENS,
                       "us": round(ms_both * 1e3, 2), "tensor_scale_us": round(ms_scale * 1e3, 2),
                       "GB/s": round(b / ms_both / 1e6, 1), "frac_hbm": round(b / ms_both / 1e6 / HBM_PEAK_GBS, 4)})
+        # the same as ONE launch (arcq_reorder_quantize_x_absmax: rows stay in LDS while the workgroups exchange maxima)
+        ms_one = time_quant(lambda i: L.arcq_reorder_quantize_x_absmax(
+            xs[i % nbuf].data_ptr(), M_TOKENS, H, idx.data_ptr(), SELECT, fid["NVFP4"], 2688.0, sc.data_ptr(), q.data_ptr(),
+            sf.data_ptr(), stream), M_TOKENS, 100)
+        b1 = quant_bytes(M_TOKENS, H, SELECT, "NVFP4", False)
+        quant.append({"op": "tensor scale and reorder_quantize_x in one launch", "fmt": "NVFP4", "select_num": SELECT, "M": M_TOKENS,
+                      "us": round(ms_one * 1e3, 2), "GB/s": round(b1 / ms_one / 1e6, 1),
+                      "frac_hbm": round(b1 / ms_one / 1e6 / HBM_PEAK_GBS, 4)})
         # the fused norm at the prefill size of benchmark configuration 4 (16384 rows, rotating inputs): the rate
         # without the ramp of a 13 us launch
         M4 = 16384

@@ -155,6 +155,20 @@ int arcq_swiglu_absmax(const void *gate, const void *up, int ld, int M, int K, f
 int arcq_tensor_scale(const void *x, const void *up, int ld, int M, int K, float divisor, float *d_scale, void *stream);
 
 /*
+ * The tensor scale and the activation quantizer under it as one call: what the reference's callers write as
+ * scale = x.abs().max() / (448 * 6) followed by reorder_quantize_x(x / scale, ...) (model/qLlamaLayer.py:73-77,
+ * kernels/src/bindings.cpp:122-163).  d_scale receives max |x| / divisor (1 for an all-zero tensor); codes and
+ * scale bytes are those of arcq_reorder_quantize_x with d_global_scale = d_scale.
+ * NVFP4 activations of up to 16 rows per CU (4096 on an MI355X) and K = 1024, 2048, 3072 or 4096 take ONE launch:
+ * the rows stay in LDS while the workgroups exchange their maxima through the stream's scratch memory
+ * (arcq_prepare_stream), so x is read once.  Everything else is arcq_tensor_scale followed by the quantizer.
+ * A workgroup that does not hear from the others in time (they share the chip with other work) takes the maximum
+ * over x by itself; the result does not depend on it.
+ */
+int arcq_reorder_quantize_x_absmax(const void *x, int M, int K, const int16_t *reorder_index, int select_num, int fmt,
+                                   float divisor, float *d_scale, void *codes, void *scales, void *stream);
+
+/*
  * Augmented-K block-scaled FP4 GEMM: C[M,N] = alpha * dq(A)[M,K'] @ dq(B)[N,K']^T, fp32
  * accumulation, bf16 output.
  * Replaces agemm.matmul (kernels/src/bindings.cpp:99-120 -> nvfp4.cu:35-132).

@@ -309,3 +309,112 @@ def test_rows_of_more_than_16384_channels(agemm, oracle, fmt, M, K, S):
     want = oracle.quantize_w(w, idx, S, fmt, gw)
     q, sf = agemm.reorder_quantize_w(dev(w), dev(idx), S, fmt=fmt, global_scale=gw)
     compare("w", q, sf, want)
+
+
+def absmax_scale(x) -> float:
+    """max|x| / 2688 by an IEEE fp32 division (model/qLlamaLayer.py:73-77), 1 for an all-zero tensor"""
+    m = x.abs().max().float() / torch.full((), 2688.0)
+    return float(m) if float(m) != 0.0 else 1.0
+
+
+@pytest.mark.parametrize("M,K,S", [(4096, 4096, 256), (1, 4096, 256), (100, 2048, 128), (1000, 3072, 64), (37, 1024, 0),
+                                   (16, 4096, 4096), (4097, 4096, 256), (9, 8192, 128), (33, 1056, 32)])
+def test_scale_and_quantize_in_one_call(agemm, oracle, M, K, S):
+    """reorder_quantize_x(global_scale="absmax"): the scale is torch's abs().max() / 2688 by an IEEE division, codes
+    and scale bytes are the oracle's under that scale -- for tensors that take the one-launch kernel (rows stay in
+    LDS while the workgroups exchange maxima) and for those that fall back to two launches (more than 4096 rows,
+    other row lengths).  Called three times in a row on one stream: the exchange leaves nothing behind."""
+    x = recipes.activations(M, K, seed=7000 + M + K + S)
+    x[M // 2, K // 3] = -913.0                                   # the maximum is a negative element of one row
+    idx = recipes.reorder_index(x)
+    gs = absmax_scale(x)
+    want = oracle.quantize_x(x, idx, S, "NVFP4", gs)
+    xd, idxd = dev(x), dev(idx)
+    print(f"scale + quantize M={M} K={K} S={S} gscale={gs}", flush=True)
+    for _ in range(3):
+        q, sf, scale = agemm.reorder_quantize_x(xd, idxd, S, fmt="NVFP4", global_scale="absmax")
+        assert scale.dtype == torch.float32 and scale.dim() == 0 and float(scale) == gs
+        compare("absmax", q, sf, want)
+
+
+def test_scale_and_quantize_special_tensors(agemm, oracle):
+    """All zeros -> scale 1; launches of different sizes one after the other on one stream; MXFP4 (no tensor scale
+    in the format: the call still returns max / 2688 and quantizes under it, as the two separate calls do)."""
+    K, S = 4096, 128
+    idx = dev(recipes.reorder_index(recipes.activations(8, K, seed=1)))
+    z = torch.zeros(48, K, dtype=torch.bfloat16, device="cuda")
+    q, sf, scale = agemm.reorder_quantize_x(z, idx, S, fmt="NVFP4", global_scale="absmax")
+    assert float(scale) == 1.0 and int(q.max()) == 0
+    for M in (4096, 17, 2048, 1, 300):
+        x = recipes.activations(M, K, seed=M)
+        gs = absmax_scale(x)
+        want = oracle.quantize_x(x, idx.cpu(), S, "NVFP4", gs)
+        print(f"scale + quantize, sizes in turn: M={M}", flush=True)
+        q, sf, scale = agemm.reorder_quantize_x(dev(x), idx, S, fmt="NVFP4", global_scale="absmax")
+        assert float(scale) == gs
+        compare(f"M={M}", q, sf, want)
+    x = recipes.activations(64, K, seed=5)
+    q, sf, scale = agemm.reorder_quantize_x(dev(x), idx, S, fmt="MXFP4", global_scale="absmax")
+    q2, sf2 = agemm.reorder_quantize_x(dev(x), idx, S, fmt="MXFP4", global_scale=scale)
+    assert float(scale) == absmax_scale(x) and torch.equal(q, q2) and torch.equal(sf, sf2)
+
+
+def test_scale_and_quantize_in_a_graph(agemm, oracle):
+    """The one-launch kernel takes nothing from the host that changes from launch to launch, so a captured launch can
+    be replayed: three replays with other input values each time, eager launches of another size in between."""
+    M, K, S = 512, 4096, 256
+    idx = dev(recipes.reorder_index(recipes.activations(8, K, seed=2)))
+    xs = [recipes.activations(M, K, seed=40 + i) * (1.0 + i) for i in range(3)]
+    buf = dev(xs[0]).clone()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        agemm.prepare_stream()
+        agemm.reorder_quantize_x(buf, idx, S, fmt="NVFP4", global_scale="absmax")   # warm-up outside the capture
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            q, sf, scale = agemm.reorder_quantize_x(buf, idx, S, fmt="NVFP4", global_scale="absmax")
+        for i, x in enumerate(xs):
+            buf.copy_(dev(x))
+            graph.replay()
+            stream.synchronize()
+            gs = absmax_scale(x)
+            print(f"graph replay {i} gscale={gs}", flush=True)
+            assert float(scale) == gs
+            compare(f"replay {i}", q, sf, oracle.quantize_x(x, idx.cpu(), S, "NVFP4", gs))
+            other = recipes.activations(33, K, seed=90 + i)
+            q2, sf2, s2 = agemm.reorder_quantize_x(dev(other), idx, S, fmt="NVFP4", global_scale="absmax")
+            stream.synchronize()
+            assert float(s2) == absmax_scale(other)
+
+
+_ALONE = r"""
+import sys, torch
+sys.path.insert(0, sys.argv[1])
+import recipes
+from arcquant_amd import agemm
+for M, K, S in ((4096, 4096, 256), (50, 2048, 64), (4096, 4096, 256)):
+    x = recipes.activations(M, K, seed=M + K).cuda()
+    idx = recipes.reorder_index(x.cpu()).cuda()
+    print("alone", M, K, S, flush=True)
+    q, sf, scale = agemm.reorder_quantize_x(x, idx, S, fmt="NVFP4", global_scale="absmax")
+    g = agemm.tensor_scale(x)
+    q2, sf2 = agemm.reorder_quantize_x(x, idx, S, fmt="NVFP4", global_scale=g)
+    torch.cuda.synchronize()
+    assert float(scale) == float(g) and torch.equal(q, q2) and torch.equal(sf, sf2), (M, K, S)
+print("ALONE-OK")
+"""
+
+
+def test_scale_and_quantize_when_the_workgroups_do_not_meet(agemm):
+    """A workgroup that does not hear from the others in time takes the tensor's maximum by itself.  With a waiting
+    time of zero (ARCQ_RESIDENT_SPIN_US=0, read when the library is first used: hence a process of its own) every
+    workgroup does so unless the others happen to be done already; results equal the two separate calls'."""
+    import os
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    env = dict(os.environ, ARCQ_RESIDENT_SPIN_US="0", PYTHONPATH=os.path.dirname(here) + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    out = subprocess.run([sys.executable, "-c", _ALONE, here], env=env, capture_output=True, text=True, timeout=300)
+    print(out.stdout[-2000:], out.stderr[-2000:], flush=True)
+    assert out.returncode == 0 and "ALONE-OK" in out.stdout
