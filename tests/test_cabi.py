@@ -51,6 +51,7 @@ def test_argument_errors_need_no_gpu(K, S, fmt, want):
     for fn in (L.arcq_reorder_quantize_x, L.arcq_reorder_quantize_w):
         assert fn(dummy, 4, K, dummy, S, fmt, 1.0, None, dummy, dummy, None) == want
     assert L.arcq_rmsnorm_quantize_x(dummy, dummy, 1e-5, 4, K, dummy, S, fmt, 1.0, None, dummy, dummy, None) == want
+    assert L.arcq_reorder_quantize_x_absmax(dummy, 4, K, dummy, S, fmt, 2688.0, dummy, dummy, dummy, None) == want
 
 
 def test_null_alignment_and_matmul_errors():
@@ -59,6 +60,11 @@ def test_null_alignment_and_matmul_errors():
     assert L.arcq_reorder_quantize_x(None, 4, 4096, ok, 0, 0, 1.0, None, ok, ok, None) == 1
     assert L.arcq_reorder_quantize_x(odd, 4, 4096, ok, 0, 0, 1.0, None, ok, ok, None) == 4
     assert L.arcq_reorder_quantize_x(ok, 0, 4096, ok, 0, 0, 1.0, None, ok, ok, None) == 0   # zero rows: nothing to do
+    absmax = L.arcq_reorder_quantize_x_absmax                                                # scale + quantizer as one call
+    assert absmax(ok, 4, 4096, ok, 0, 0, 2688.0, None, ok, ok, None) == 1                    # nowhere to put the scale
+    assert absmax(None, 4, 4096, ok, 0, 0, 2688.0, ok, ok, ok, None) == 1
+    assert absmax(odd, 4, 4096, ok, 0, 0, 2688.0, ok, ok, ok, None) == 4
+    assert absmax(ok, 4, 4096, ok, 0, 0, 0.0, ok, ok, ok, None) == 2                         # divisor must be positive
     assert L.arcq_matmul(ok, ok, ok, ok, 4, 4, 100, 0, 1.0, None, None, ok, None) == 2       # K' % 64
     assert L.arcq_matmul(ok, ok, ok, ok, 4, 4, 128, 5, 1.0, None, None, ok, None) == 3
     assert L.arcq_matmul(ok, None, ok, ok, 4, 4, 128, 0, 1.0, None, None, ok, None) == 1
