@@ -1065,8 +1065,9 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_wave_kernel(Quan
 // quantizer (model/qLlamaLayer.py:73-77): two passes over x.  Here a wave loads its row into LDS once, the
 // workgroups exchange their maxima, and the rows are encoded from LDS under the scale.
 //
-// Exchange: workgroup b stores (tag, maximum) as one 64-bit word into slot b; wave 0 of every workgroup reads all
-// slots until each carries the launch's tag.  The tag is one more than the value of an epoch word read at the
+// Exchange: workgroup b stores (tag, maximum) as one 64-bit word into slot b (48 bits of tag; the maximum is a bf16
+// value, its upper 16 bits say everything); wave 0 of every workgroup reads all slots until each carries the
+// launch's tag.  The tag is one more than the value of an epoch word read at the
 // start; on its way out every workgroup raises the epoch word to its tag (atomic maximum), so the next launch on
 // the stream -- which starts after this one has ended -- takes a tag above every tag ever stored.  No counter to
 // reset, no read-modify-write on the way in, nothing the host has to pass: a captured launch replays correctly.
@@ -1078,7 +1079,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_wave_kernel(Quan
 // ---------------------------------------------------------------------------------------------
 constexpr int kResidentSlots = 256;        // workgroups per launch at most (512 of half the size: 2 us slower at 2048 rows)
 constexpr int kResidentSlotWord = 256;     // slots start at this 64-bit word of the tensor-scale scratch (byte 2048)
-constexpr int kResidentEpochWord = 480;   // 32-bit word of the epoch, on a 128-byte line of its own behind the
+constexpr int kResidentEpochWord = 480;   // 32-bit word index of the 64-bit epoch, on a 128-byte line of its own behind the
                                           // (maximum, counter) pairs of tensor_scale_kernel
 
 typedef uint16_t v2u16 __attribute__((ext_vector_type(2)));
@@ -1118,7 +1119,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(
   const int row = blockIdx.x * RPW + r_in;
   const bool has_row = row < p.rows;
   unsigned long long *slots = reinterpret_cast<unsigned long long *>(ws) + kResidentSlotWord;
-  uint32_t *epoch = ws + kResidentEpochWord;
+  unsigned long long *epoch = reinterpret_cast<unsigned long long *>(ws + kResidentEpochWord);
   const uint16_t *src = p.x + (size_t)row * K + sub * CPW * 512;
   const uint32_t dst = slot_addr + sub * CPW * 1024;
 
@@ -1130,8 +1131,8 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(
     const uint8_t *g = reinterpret_cast<const uint8_t *>(p.idx) + 1024 * wave + 16 * lane;
     row_dma16<0>(g, lds0 + 1024 * wave);
   }
-  uint32_t tag = 0u;
-  if (wave == 0) tag = __hip_atomic_load(epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;  // every lane: uniform
+  unsigned long long tag = 0ull;
+  if (wave == 0) tag = __hip_atomic_load(epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1ull;  // every lane: uniform
   if (early) wait_vm<CPW>();
   else wait_vm<0>();
   lds_barrier();
@@ -1204,7 +1205,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(
     }
     wg = __builtin_amdgcn_readfirstlane(wg);
     if (lane == 0)
-      __hip_atomic_store(slots + blockIdx.x, ((unsigned long long)tag << 32) | wg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(slots + blockIdx.x, (tag << 16) | (wg >> 16), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (WPR != 1) gather_units();  // while the slot is on its way
   if (wave == 0) {
@@ -1222,8 +1223,8 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(
       for (int j = 0; j < kResidentSlots / 64; ++j) {
         if (pending & (1u << j)) {
           const unsigned long long v = __hip_atomic_load(slots + lane + 64 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if ((uint32_t)(v >> 32) == tag) {
-            const uint32_t mv = (uint32_t)v;
+          if ((v >> 16) == tag) {
+            const uint32_t mv = ((uint32_t)v & 0xffffu) << 16;
             all = mv > all ? mv : all;
             pending &= ~(1u << j);
           }
