@@ -1089,11 +1089,28 @@ __device__ __forceinline__ uint32_t absmax_bf16_pairs(uint32_t m, uint32_t w) {
   return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));  // v_pk_max_u16
 }
 
+// Compile-time loop over 0 .. N-1 and a choice among four arrays by a compile-time index: the units' values live in
+// four separate arrays of sixteen registers (one array of 64 stays in scratch memory: the compiler does not split it).
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+template <int U>
+__device__ __forceinline__ uint32_t (&pick16(uint32_t (&a)[16], uint32_t (&b)[16], uint32_t (&c)[16], uint32_t (&d)[16]))[16] {
+  if constexpr (U == 0) return a;
+  else if constexpr (U == 1) return b;
+  else if constexpr (U == 2) return c;
+  else return d;
+}
+
 // WPR waves share a row (1, 2 or 4: a row's units are dealt out to them by whole rounds of 64), so that a launch of
 // few rows still spreads over the chip: a workgroup holds 16 / WPR rows, and a wave's share of the arithmetic that
 // follows the exchange -- where nothing else can hide it -- is 1 / WPR of a row.
 template <int FMT, int KU, int WPR>
-__global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(QuantParams p, float divisor, uint32_t spin_ticks,
+__global__ __launch_bounds__(64 * kRowWaves) __attribute__((amdgpu_waves_per_eu(4, 4))) void quantize_rows_resident_kernel(QuantParams p, float divisor, uint32_t spin_ticks,
                                                                                  uint32_t *ws, float *scale_out) {
   extern __shared__ uint4 smem[];
   constexpr int G = FMT == ARCQ_FMT_NVFP4 ? 16 : 32;
@@ -1141,11 +1158,9 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(
 
   // what does not depend on the scale: the maximum, and the units' values in the channel order
   uint32_t m = 0u;
-  uint32_t yp[UPL][8];
+  uint32_t ya[16], yb[16], yc[16], yd[16];  // fp32 bits: a bf16 loaded into the upper half of a zeroed register IS the fp32
 #pragma unroll
-  for (int u = 0; u < UPL; ++u)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) yp[u][j] = 0u;
+  for (int k = 0; k < 16; ++k) ya[k] = yb[k] = yc[k] = yd[k] = 0u;
   if (has_row) {
 #pragma unroll
     for (int c = 0; c < CPW; ++c) {
@@ -1153,15 +1168,11 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(
       m = absmax_bf16_pairs(absmax_bf16_pairs(absmax_bf16_pairs(absmax_bf16_pairs(m, q.x), q.y), q.z), q.w);
     }
   }
-  // A 16-bit LDS load into one half of a register clears the other half on this chip, so two channels cannot be
-  // loaded into one register: sixteen registers per unit (high halves), then one byte permute per pair.
   auto gather_units = [&]() {
     if (!has_row) return;
     const uint4 *idx_t = reinterpret_cast<const uint4 *>(lds);
-    uint32_t ta[16], tb[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) ta[i] = tb[i] = 0u;
-    auto request = [&](int u, uint32_t (&t)[16]) {
+    static_for<UPL>([&](auto U) {
+      constexpr int u = decltype(U)::value;
       const int n = (sub * UPL + u) * 64 + lane;
       const uint4 i0 = idx_t[2 * n], i1 = idx_t[2 * n + 1];
       const uint32_t iw[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
@@ -1171,20 +1182,14 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(
         addr[2 * j] = gather_addr<0>(iw[j], slot_addr);
         addr[2 * j + 1] = gather_addr<1>(iw[j], slot_addr);
       }
-      gather16(t, addr);
-    };
-    request(0, ta);
+      gather16(pick16<u>(ya, yb, yc, yd), addr);
+    });
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    static_for<UPL>([&](auto U) {
+      uint32_t(&v)[16] = pick16<decltype(U)::value>(ya, yb, yc, yd);
 #pragma unroll
-    for (int u = 0; u < UPL; ++u) {
-      uint32_t(&cur)[16] = (u & 1) ? tb : ta;
-      uint32_t(&nxt)[16] = (u & 1) ? ta : tb;
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-      for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(cur[i]));  // read after the wait above
-#pragma unroll
-      for (int j = 0; j < 8; ++j) yp[u][j] = __builtin_amdgcn_perm(cur[2 * j + 1], cur[2 * j], 0x07060302u);
-      if (u + 1 < UPL) request(u + 1, nxt);
-    }
+      for (int k = 0; k < 16; ++k) asm volatile("" : "+v"(v[k]));  // read after the wait above
+    });
   };
   if (WPR == 1) gather_units();  // the row is this wave's own: no need to wait for anybody
   m = (m & 0xffffu) > (m >> 16) ? (m << 16) : (m & 0xffff0000u);  // the larger half, as the bits of an fp32
@@ -1279,22 +1284,16 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_resident_kernel(
   const bool g_odd = !(fabsf(g) >= 0x1p-60f && fabsf(g) <= 0x1p+60f);
   const bool coarse = (f2u(g) & 0x7fffffu) == 0u;
   uint8_t *crow = p.codes + (size_t)row * (Kp >> 1), *srow = p.scales + (size_t)row * (Kp / G);
-#pragma unroll
-  for (int u = 0; u < UPL; ++u) {
-    uint32_t yv[16];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      yv[2 * j] = yp[u][j] << 16;
-      yv[2 * j + 1] = yp[u][j] & 0xffff0000u;
-    }
+  static_for<UPL>([&](auto U) {
+    constexpr int u = decltype(U)::value;
     const int n = (sub * UPL + u) * 64 + lane;
     const bool tail = n >= tail0;
     uint2 pk, pk2;
     uint32_t sb, sb2;
-    quantize_unit<FMT, MODE_X, true>(yv, true, tail, g, rg, g_odd, coarse, pk, sb, pk2, sb2);
+    quantize_unit<FMT, MODE_X, true>(pick16<u>(ya, yb, yc, yd), true, tail, g, rg, g_odd, coarse, pk, sb, pk2, sb2);
     store_unit<FMT>(crow, srow, n, pk, sb);
     if (tail) store_unit<FMT>(crow, srow, nunits + (n - tail0), pk2, sb2);
-  }
+  });
 }
 
 // max |act_fn(gate) * up| over the whole tensor (the NVFP4 tensor scale's numerator,
