@@ -415,21 +415,45 @@ __device__ __forceinline__ void quantize_unit(const uint32_t (&yv)[16], bool act
 #pragma unroll
   for (int i = 0; i < 16; ++i) y[i] = u2f(yv[i]);
   if (SCALED) {
-    // A tensor scale that is not a power of two, and no lane of the wave has a residual to form (those need
-    // y = x / g itself): one division per unit.  RN(x / g) is monotone in |x|, so the block maximum of y is the
-    // quotient of the block maximum of x; the codes come straight from x (encode_unit_two_sided_x).
-    const bool wave_has_tail = MODE != MODE_W && __builtin_amdgcn_ballot_w64(tail) != 0ull;
-    if (!coarse && !wave_has_tail) {
+    // A tensor scale that is not a power of two: one division per unit for the main block.  RN(x / g) is monotone in
+    // |x|, so the block maximum of y is the quotient of the block maximum of x; the codes come straight from x
+    // (encode_unit_two_sided_x).  Only a wave that holds residual units forms y = x / g itself, for the residual.
+    if (!coarse) {
       float s;
       const float amax = div_bf16_by(unit_amax3<FMT>(y), g, rg);
       const float t = div6_any(amax);
       sb = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t, &s) : ue8m0_scale(t, &s);
       pk = encode_unit_two_sided_x(y, g, rg, s, rg * scale_rcp<FMT>(s));
       bool redo = amax_needs_exact(amax) || g_odd;
-      if (FMT == ARCQ_FMT_MXFP4) redo = __shfl_xor((int)redo, 1) != 0 || redo;
-      if (redo && active) unit_exact<FMT, false>(yv, g, &pk, &sb, &pk2, &sb2);
       pk2 = pk;
       sb2 = sb;
+      const bool wave_has_tail = MODE != MODE_W && __builtin_amdgcn_ballot_w64(tail) != 0ull;
+      if (wave_has_tail) {
+        float e[16];
+        decode_unit(pk, e);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) e[i] = __builtin_fmaf(-e[i], s, div_bf16_by(y[i], g, rg));  // the fp32 residual y - q*s
+        float s2;
+        const float amax2 = unit_amax3<FMT>(e);
+        const float t2 = div6_any(amax2);
+        const uint32_t sbr = FMT == ARCQ_FMT_NVFP4 ? ue4m3_scale(t2, &s2) : ue8m0_scale(t2, &s2);
+        const uint2 pkr = encode_unit_two_sided(e, s2, scale_rcp<FMT>(s2));
+        if (tail) {
+          pk2 = pkr;
+          sb2 = sbr;
+          redo = amax_needs_exact(amax2) || redo;
+        }
+      }
+      if (FMT == ARCQ_FMT_MXFP4) redo = __shfl_xor((int)redo, 1) != 0 || redo;  // both halves of a 32-block
+      if (redo && active) {
+        if (MODE != MODE_W && tail) {
+          unit_exact<FMT, true>(yv, g, &pk, &sb, &pk2, &sb2);
+        } else {
+          unit_exact<FMT, false>(yv, g, &pk, &sb, &pk2, &sb2);
+          pk2 = pk;
+          sb2 = sb;
+        }
+      }
       return;
     }
 #pragma unroll
