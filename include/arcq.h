@@ -55,9 +55,11 @@ int arcq_last_hip_error(void);
 /*
  * Scratch memory.  Three kernels need device memory beyond their inputs and outputs: the split-K GEMM
  * (fp32 partial tiles, arcq_matmul on narrow layers with few rows), the split decode attention
- * (partial softmax sums, arcq_kv_decode_i4 with few sequences) and arcq_tensor_scale (two words).
+ * (partial softmax sums, arcq_kv_decode_i4 with few sequences) and arcq_tensor_scale /
+ * arcq_reorder_quantize_x_absmax (a few words and one 8-byte slot per workgroup, through which the workgroups of a
+ * launch exchange their maxima; zeroed once, every launch leaves them ready for the next).
  * The library keeps one buffer of each kind per (device, stream), allocated on the first call that
- * needs it and kept until arcq_release_stream or the end of the process (32 MiB + 8 MiB + 2 KiB when all
+ * needs it and kept until arcq_release_stream or the end of the process (32 MiB + 8 MiB + 4 KiB when all
  * three exist); calls on one stream are serialised, so they never share a buffer with a call on another
  * stream.  An allocation cannot happen while the stream is being captured into a
  * graph: such a call returns ARCQ_ERR_WORKSPACE unless the stream has its buffers already.
