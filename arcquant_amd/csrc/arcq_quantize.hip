@@ -1973,7 +1973,16 @@ int arcq_reorder_quantize_x_absmax(const void *x, int M, int K, const int16_t *r
   if (!d_scale || (M > 0 && (!x || !reorder_index || !codes || !scales))) return ARCQ_ERR_NULL;
   if (M > 0 && (!arcq::aligned16(x) || !arcq::aligned16(reorder_index) || !arcq::aligned16(codes))) return ARCQ_ERR_ALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (M > 0 && fmt == ARCQ_FMT_NVFP4 && arcq::tuning().resident_spin_us >= 0) {
+  if (M == 0) {  // an empty tensor: nothing to quantize, scale 1 (one workgroup of the scale kernel over no rows)
+    int status = ARCQ_OK;
+    uint32_t *ws = static_cast<uint32_t *>(arcq::stream_workspace(arcq::kWsTensorScale, st, &status));
+    if (!ws) return status;
+    hipLaunchKernelGGL(arcq::tensor_scale_kernel<false>, dim3(1), dim3(512), 0, st, static_cast<const uint16_t *>(nullptr),
+                       static_cast<const uint16_t *>(nullptr), (size_t)K, 0, K, divisor, ws, d_scale);
+    ARCQ_HIP_TRY(hipGetLastError());
+    return ARCQ_OK;
+  }
+  if (fmt == ARCQ_FMT_NVFP4 && arcq::tuning().resident_spin_us >= 0) {
     arcq::QuantParams p;
     p.x = static_cast<const uint16_t *>(x);
     p.gamma = nullptr;
@@ -1993,7 +2002,7 @@ int arcq_reorder_quantize_x_absmax(const void *x, int M, int K, const int16_t *r
     if (rc >= 0) return rc;
   }
   // tensors beyond the chip's LDS, other row lengths, MXFP4: the scale, then the quantizer under it
-  const int rc = arcq_tensor_scale(x ? x : d_scale, nullptr, K, M, K, divisor, d_scale, stream);
+  const int rc = arcq_tensor_scale(x, nullptr, K, M, K, divisor, d_scale, stream);
   if (rc != ARCQ_OK) return rc;
   return arcq::quantize_entry(arcq::MODE_X, x, nullptr, 0.0f, M, K, reorder_index, select_num, fmt, 1.0f, d_scale, codes, scales,
                               stream);

@@ -345,6 +345,8 @@ def test_scale_and_quantize_special_tensors(agemm, oracle):
     z = torch.zeros(48, K, dtype=torch.bfloat16, device="cuda")
     q, sf, scale = agemm.reorder_quantize_x(z, idx, S, fmt="NVFP4", global_scale="absmax")
     assert float(scale) == 1.0 and int(q.max()) == 0
+    q, sf, scale = agemm.reorder_quantize_x(z[:0], idx, S, fmt="NVFP4", global_scale="absmax")   # no rows at all
+    assert q.shape == (0, (K + S) // 2) and sf.numel() == 0 and float(scale) == 1.0
     for M in (4096, 17, 2048, 1, 300):
         x = recipes.activations(M, K, seed=M)
         gs = absmax_scale(x)
