@@ -1086,8 +1086,9 @@ __global__ __launch_bounds__(64 * kRowWaves) void quantize_rows_wave_kernel(Quan
 // ---------------------------------------------------------------------------------------------
 // Tensor scale and quantizer in one launch, for activations that fit the chip's LDS (sixteen rows of up to 4096
 // channels per CU: 4096 rows on 256 CUs).  The reference's callers form max|x| / 2688 with torch ahead of the
-// quantizer (model/qLlamaLayer.py:73-77): two passes over x.  Here a wave loads its row into LDS once, the
-// workgroups exchange their maxima, and the rows are encoded from LDS under the scale.
+// quantizer (model/qLlamaLayer.py:73-77): two passes over x.  Here a wave loads its row into LDS once, takes its
+// maximum and gathers its units into registers in the channel order; the workgroups exchange their maxima; then
+// the units are encoded under the scale.
 //
 // Exchange: workgroup b stores (tag, maximum) as one 64-bit word into slot b (48 bits of tag; the maximum is a bf16
 // value, its upper 16 bits say everything); wave 0 of every workgroup reads all slots until each carries the
